@@ -1,0 +1,142 @@
+/* tri_attn.h — C ABI of libtrident_attn.so: scaled-dot-product attention forward and backward
+ * for one MI355X (gfx950).
+ *
+ * This library replaces the three Triton launches of the reference's attention operation:
+ *   kernel.Attention.forward       launched at trident/operation/attention.py:109-131
+ *   kernel.Softmax.backward_delta  launched at trident/operation/attention.py:161-163
+ *   kernel.Attention.backward      launched at trident/operation/attention.py:170-199
+ * (kernel argument lists: trident/kernel/attention.py:33-56 and :169-197,
+ *  trident/kernel/softmax.py:184-193).
+ *
+ * Conventions
+ *   - Every pointer is a device pointer owned by the caller; the library never allocates or
+ *     frees memory and never synchronises the device. Work is enqueued on `stream`
+ *     (a hipStream_t; NULL = the default stream) and the buffers must stay alive until the
+ *     stream has passed the call.
+ *   - Tensors are [B, H, S, D] with element strides given for all four dimensions.
+ *     The innermost (D) stride of q, k, v, o, d_o, dq, dk, dv must be 1.
+ *   - lse and delta are dense fp32 [B, H, S]. lse holds log2(sum_j exp(s_ij)) with
+ *     s = q k^T * softmax_scale + mask, i.e. natural-log LSE times log2(e)
+ *     (the same log2-domain statistic the reference saves, trident/kernel/attention.py:164,
+ *     but always fp32).
+ *   - mask is additive, dtype mask_dtype, logical shape [B, H, S, S] with element strides;
+ *     a stride of 0 broadcasts that dimension; the innermost mask stride must be 1.
+ *     mask and is_causal are mutually exclusive (trident/operation/attention.py:41-43).
+ *   - Causal rule: key j is visible to query i iff i >= j (trident/kernel/attention.py:131-134).
+ *   - Dropout acts on the probabilities: P is multiplied by keep/(1 - thr8/256) where
+ *     thr8 = clamp(rint(dropout_p * 256), 0, 256) and keep comes from Philox4x32-10:
+ *       key = (seed & 0xffffffff, seed >> 32); ctr = (j >> 2, i >> 2, b*H + h, offset);
+ *       u8 = (r[i & 3] >> (8 * (j & 3))) & 0xff; keep = u8 >= thr8.
+ *     The backward calls must be given the same seed, offset and dropout_p as the forward.
+ *   - All entry points return 0 on success, a negative TRI_ATTN_E* code for an argument
+ *     error, or a positive hipError_t if a launch failed. They are re-entrant and keep no
+ *     mutable global state.
+ */
+#ifndef TRI_ATTN_H
+#define TRI_ATTN_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TRI_ATTN_ABI_VERSION 1
+
+enum {
+    TRI_ATTN_F32 = 0,
+    TRI_ATTN_F16 = 1,
+    TRI_ATTN_BF16 = 2
+};
+
+enum {
+    TRI_ATTN_OK = 0,
+    TRI_ATTN_ENULL = -1,      /* a required pointer is NULL */
+    TRI_ATTN_ESHAPE = -2,     /* B,H,S,D out of range or D not in {16,32,64,128} */
+    TRI_ATTN_EDTYPE = -3,     /* unknown dtype / mask_dtype */
+    TRI_ATTN_ESTRIDE = -4,    /* innermost stride is not 1, or a stride is negative */
+    TRI_ATTN_EMASKCAUSAL = -5,/* both mask and is_causal set */
+    TRI_ATTN_EDROPOUT = -6,   /* dropout_p outside [0,1] */
+    TRI_ATTN_ESIZE = -7,      /* struct_size does not match this ABI version */
+    TRI_ATTN_EALIGN = -8      /* a pointer or stride breaks the 16-byte alignment the kernels need */
+};
+
+typedef struct TriAttnArgs {
+    uint32_t struct_size;      /* = sizeof(TriAttnArgs) */
+    int32_t dtype;             /* TRI_ATTN_F32 / F16 / BF16: element type of q,k,v,o,d_o,dq,dk,dv */
+    int32_t B, H, S, D;        /* y_size = S, x_size = D in the reference's naming */
+    int32_t is_causal;
+    int32_t mask_dtype;        /* element type of mask and dmask */
+    float softmax_scale;
+    float dropout_p;
+    uint64_t seed;             /* Philox key */
+    uint64_t offset;           /* Philox counter word 3 (low 32 bits used) */
+
+    const void* q;             /* query  (query_ptr) */
+    const void* k;             /* key    (key_ptr) */
+    const void* v;             /* value  (value_ptr) */
+    void* o;                   /* output (output_ptr); input to the backward calls */
+    float* lse;                /* log2sum_ptr, fp32 [B,H,S]; written by fwd, read by bwd */
+    const void* mask;          /* mask_ptr or NULL */
+    const void* d_o;           /* grad_output_ptr */
+    void* dq;                  /* grad_query_ptr (need not be zeroed) */
+    void* dk;                  /* grad_key_ptr */
+    void* dv;                  /* grad_value_ptr */
+    void* dmask;               /* grad_mask_ptr or NULL: dense [B,H,S,S] in mask_dtype, dS per head */
+    float* delta;              /* delta_ptr, fp32 [B,H,S]: written by bwd_delta, read by dkdv/dq */
+
+    int64_t q_stride[4];
+    int64_t k_stride[4];
+    int64_t v_stride[4];
+    int64_t o_stride[4];
+    int64_t do_stride[4];
+    int64_t dq_stride[4];
+    int64_t dk_stride[4];
+    int64_t dv_stride[4];
+    int64_t mask_stride[4];
+    int64_t dmask_stride[4];
+
+    void* stream;              /* hipStream_t */
+} TriAttnArgs;
+
+/* ABI version of the loaded library (TRI_ATTN_ABI_VERSION it was built with). */
+int tri_attn_version(void);
+
+/* Text for a status code returned by any entry point below. */
+const char* tri_attn_strerror(int status);
+
+/* Replaces kernel.Attention.forward (trident/kernel/attention.py:33-165; launch at
+ * trident/operation/attention.py:109-131). Reads q,k,v[,mask]; writes o and lse. */
+int tri_attn_fwd(const TriAttnArgs* args);
+
+/* Replaces kernel.Softmax.backward_delta as attention uses it (trident/kernel/softmax.py:184-238;
+ * launch at trident/operation/attention.py:161-163). Reads o, d_o; writes delta = rowsum(d_o * o). */
+int tri_attn_bwd_delta(const TriAttnArgs* args);
+
+/* First half of kernel.Attention.backward (trident/kernel/attention.py:169-339; launch at
+ * trident/operation/attention.py:170-199): dK and dV, one workgroup per key tile.
+ * Reads q,k,v,d_o,lse,delta[,mask]; writes dk, dv. */
+int tri_attn_bwd_dkdv(const TriAttnArgs* args);
+
+/* Second half of kernel.Attention.backward: dQ (and dMask when args->dmask is set), one
+ * workgroup per query tile, so every dQ tile is written once and needs no zero fill
+ * (the reference accumulates into a zeroed dQ, trident/kernel/attention.py:321-323).
+ * Reads q,k,v,d_o,lse,delta[,mask]; writes dq[, dmask]. */
+int tri_attn_bwd_dq(const TriAttnArgs* args);
+
+/* The whole backward in launch order: bwd_delta, bwd_dkdv, bwd_dq
+ * (trident/operation/attention.py:137-202). */
+int tri_attn_bwd(const TriAttnArgs* args);
+
+/* Debug / parity helper with no counterpart in the reference (its dropout stream is unpinned):
+ * writes the dropout keep decisions (1 = kept) for head index bh, rows [row0,row0+rows),
+ * cols [col0,col0+cols) into keep[rows*cols] (device, uint8) using exactly the device code
+ * the attention kernels use. */
+int tri_attn_dropout_mask(uint64_t seed, uint64_t offset, float dropout_p, uint32_t bh,
+                          int32_t row0, int32_t rows, int32_t col0, int32_t cols,
+                          uint8_t* keep, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRI_ATTN_H */

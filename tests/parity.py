@@ -1,0 +1,46 @@
+"""Shared helpers of the parity tests: oracle calls on torch tensors and the comparison rule."""
+import numpy as np
+import torch
+
+from oracle import attention as oracle
+
+# north_star tolerances: fp32 atol 1e-4; fp16/bf16 atol 1e-2 against an fp32/fp64 reference.
+ATOL = {torch.float32: 1e-4, torch.float16: 1e-2, torch.bfloat16: 1e-2}
+# A correctly rounded result in a 16-bit type is itself off by up to half an ulp of the output
+# (2^-9 relative for bf16, 2^-12 for fp16), which exceeds 1e-2 once |x| > 4 in bf16. That
+# storage rounding is added to the tolerance; the arithmetic error budget stays atol.
+RTOL = {torch.float32: 1e-5, torch.float16: 2.0**-11, torch.bfloat16: 2.0**-8}
+
+
+def to64(t):
+    return None if t is None else t.detach().cpu().to(torch.float64).numpy()
+
+
+def close(actual: torch.Tensor, expected: np.ndarray, dtype, what=""):
+    a = actual.detach().cpu().to(torch.float64).numpy()
+    e = np.asarray(expected, dtype=np.float64)
+    assert a.shape == e.shape, (what, a.shape, e.shape)
+    both_nan = np.isnan(a) & np.isnan(e)
+    err = np.abs(a - e)
+    err[both_nan] = 0.0
+    tol = ATOL[dtype] + RTOL[dtype] * np.abs(e)
+    tol = np.where(np.isfinite(tol), tol, np.inf)
+    bad = ~(err <= tol)
+    bad &= ~((a == e) & ~np.isnan(a))  # equal infinities
+    if bad.any():
+        idx = np.unravel_index(np.argmax(np.where(bad, err, 0)), a.shape)
+        raise AssertionError(
+            f"{what}: {bad.sum()} of {a.size} elements off; worst at {idx}: got {a[idx]!r}, want {e[idx]!r}, "
+            f"max abs err {np.nanmax(err):.3e}"
+        )
+    return float(np.nanmax(err)) if err.size else 0.0
+
+
+def oracle_forward(q, k, v, mask=None, dropout_p=0.0, is_causal=False, scale=None, seed=0, offset=0):
+    return oracle.attention_forward(to64(q), to64(k), to64(v), to64(mask), dropout_p, is_causal, scale, seed, offset)
+
+
+def oracle_backward(q, k, v, d_o, mask=None, dropout_p=0.0, is_causal=False, scale=None, seed=0, offset=0,
+                    want_dmask=False):
+    return oracle.attention_backward(to64(q), to64(k), to64(v), to64(d_o), to64(mask), dropout_p, is_causal, scale,
+                                     seed, offset, want_dmask)

@@ -1,0 +1,111 @@
+"""Boundary checks that need no GPU: the library loads, exports what include/tri_attn.h declares,
+the ctypes struct matches the C one, and argument errors surface as the reference's errors."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+import torch
+
+import trident_amd as trident
+from trident_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "tri_attn.h")
+
+
+def test_library_exports_every_declared_symbol():
+    text = open(HEADER).read()
+    declared = set(re.findall(r"\b(tri_attn_\w+)\s*\(", text))
+    assert declared == set(_lib.EXPORTS)
+    lib = _lib.lib()
+    for name in declared:
+        assert hasattr(lib, name)
+    assert lib.tri_attn_version() == _lib.ABI_VERSION
+
+
+def test_struct_layout_matches_header(tmp_path):
+    src = tmp_path / "sz.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <stddef.h>\n#include "tri_attn.h"\n'
+        'int main(){printf("%zu %zu %zu %zu %zu", sizeof(TriAttnArgs), offsetof(TriAttnArgs,seed),'
+        ' offsetof(TriAttnArgs,q), offsetof(TriAttnArgs,mask_stride), offsetof(TriAttnArgs,stream));}'
+    )
+    exe = tmp_path / "sz"
+    subprocess.check_call(["gcc", "-I", os.path.dirname(HEADER), str(src), "-o", str(exe)])
+    got = [int(x) for x in subprocess.check_output([str(exe)]).split()]
+    T = _lib.TriAttnArgs
+    assert got == [ctypes.sizeof(T), T.seed.offset, T.q.offset, T.mask_stride.offset, T.stream.offset]
+
+
+def test_status_codes_without_gpu():
+    lib = _lib.lib()
+    assert lib.tri_attn_fwd(None) == -1
+    args = _lib.TriAttnArgs()
+    assert lib.tri_attn_fwd(ctypes.byref(args)) == -7  # struct_size unset
+    args.struct_size = ctypes.sizeof(args)
+    args.dtype = 9
+    assert lib.tri_attn_fwd(ctypes.byref(args)) == -3
+    args.dtype = 2
+    args.B, args.H, args.S, args.D = 1, 1, 128, 48
+    assert lib.tri_attn_fwd(ctypes.byref(args)) == -2
+    args.D = 64
+    args.dropout_p = 1.5
+    assert lib.tri_attn_bwd(ctypes.byref(args)) == -6
+    args.dropout_p = 0.0
+    assert lib.tri_attn_fwd(ctypes.byref(args)) == -1  # pointers missing
+    args.mask = 64
+    args.is_causal = 1
+    assert lib.tri_attn_fwd(ctypes.byref(args)) == -5
+    assert b"mask and is_causal" in lib.tri_attn_strerror(-5)
+    assert lib.tri_attn_dropout_mask(0, 0, 0.1, 0, 0, 4, 0, 4, None, None) == -1
+
+
+def test_reference_value_errors():
+    """Same texts as trident/operation/attention.py:28-45."""
+    f = trident.function.scaled_dot_product_attention
+    x = torch.zeros(2, 4, 8, 16)
+    with pytest.raises(ValueError, match="The dimension of query, key and value should be 4."):
+        f(x[0], x[0], x[0])
+    y = torch.zeros(2, 4, 12, 16)
+    with pytest.raises(ValueError, match="Attention supports only for power of 2 size tensors."):
+        f(y, y, y)
+    m = torch.zeros(2, 4, 8, 8)
+    with pytest.raises(ValueError, match="Error because both attn_mask and is_causal are set."):
+        f(x, x, x, attn_mask=m, is_causal=True)
+    with pytest.raises(ValueError, match="Boolean mask is not supported yet."):
+        f(x, x, x, attn_mask=m.bool())
+    with pytest.raises(AssertionError):
+        z = torch.zeros(1, 1, 8, 256)
+        f(z, z, z)
+    with pytest.raises(ValueError, match="Unable to convert the given input"):
+        trident.util.dtype(torch.int8)
+
+
+def test_no_cpu_fallback():
+    x = torch.zeros(1, 1, 8, 16)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        trident.function.scaled_dot_product_attention(x, x, x)
+
+
+def test_api_surface():
+    import inspect
+
+    sig = inspect.signature(trident.function.scaled_dot_product_attention)
+    assert list(sig.parameters) == ["query", "key", "value", "attn_mask", "dropout_p", "is_causal", "use_accelerator"]
+    sig = inspect.signature(trident.function.attention)
+    assert list(sig.parameters) == ["query", "key", "value", "mask", "dropout_p", "is_causal", "softmax_scale"]
+    assert issubclass(trident.operation.Attention, torch.autograd.Function)
+    assert isinstance(trident.Attention(is_causal=True), torch.nn.Module)
+    assert trident.util.is_pow2(64) and not trident.util.is_pow2(0) and not trident.util.is_pow2(48)
+    assert trident.config.use_trace is False
+
+
+def test_product_does_not_import_oracle():
+    pkg = os.path.join(ROOT, "trident_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for name in files:
+            if name.endswith((".py", ".hip", ".hpp", ".h")):
+                text = open(os.path.join(dirpath, name)).read()
+                assert "oracle" not in text, os.path.join(dirpath, name)

@@ -1,0 +1,99 @@
+"""ctypes binding of libtrident_attn.so (declarations: include/tri_attn.h)."""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libtrident_attn.so")
+ABI_VERSION = 1
+
+_i64x4 = ctypes.c_int64 * 4
+
+
+class TriAttnArgs(ctypes.Structure):
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("dtype", ctypes.c_int32),
+        ("B", ctypes.c_int32),
+        ("H", ctypes.c_int32),
+        ("S", ctypes.c_int32),
+        ("D", ctypes.c_int32),
+        ("is_causal", ctypes.c_int32),
+        ("mask_dtype", ctypes.c_int32),
+        ("softmax_scale", ctypes.c_float),
+        ("dropout_p", ctypes.c_float),
+        ("seed", ctypes.c_uint64),
+        ("offset", ctypes.c_uint64),
+        ("q", ctypes.c_void_p),
+        ("k", ctypes.c_void_p),
+        ("v", ctypes.c_void_p),
+        ("o", ctypes.c_void_p),
+        ("lse", ctypes.c_void_p),
+        ("mask", ctypes.c_void_p),
+        ("d_o", ctypes.c_void_p),
+        ("dq", ctypes.c_void_p),
+        ("dk", ctypes.c_void_p),
+        ("dv", ctypes.c_void_p),
+        ("dmask", ctypes.c_void_p),
+        ("delta", ctypes.c_void_p),
+        ("q_stride", _i64x4),
+        ("k_stride", _i64x4),
+        ("v_stride", _i64x4),
+        ("o_stride", _i64x4),
+        ("do_stride", _i64x4),
+        ("dq_stride", _i64x4),
+        ("dk_stride", _i64x4),
+        ("dv_stride", _i64x4),
+        ("mask_stride", _i64x4),
+        ("dmask_stride", _i64x4),
+        ("stream", ctypes.c_void_p),
+    ]
+
+
+EXPORTS = (
+    "tri_attn_version",
+    "tri_attn_strerror",
+    "tri_attn_fwd",
+    "tri_attn_bwd_delta",
+    "tri_attn_bwd_dkdv",
+    "tri_attn_bwd_dq",
+    "tri_attn_bwd",
+    "tri_attn_dropout_mask",
+)
+
+_lib = None
+
+
+def lib():
+    """The loaded library. Raises if it has not been built: there is no fallback path."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m trident_amd.build` "
+                "(hipcc, gfx950). trident_amd has no CPU or PyTorch fallback."
+            )
+        cdll = ctypes.CDLL(LIB_PATH)
+        for name in EXPORTS:
+            getattr(cdll, name)  # AttributeError if a declared symbol is not exported
+        cdll.tri_attn_version.restype = ctypes.c_int
+        cdll.tri_attn_strerror.restype = ctypes.c_char_p
+        cdll.tri_attn_strerror.argtypes = [ctypes.c_int]
+        for name in ("tri_attn_fwd", "tri_attn_bwd_delta", "tri_attn_bwd_dkdv", "tri_attn_bwd_dq", "tri_attn_bwd"):
+            fn = getattr(cdll, name)
+            fn.restype = ctypes.c_int
+            fn.argtypes = [ctypes.POINTER(TriAttnArgs)]
+        cdll.tri_attn_dropout_mask.restype = ctypes.c_int
+        cdll.tri_attn_dropout_mask.argtypes = [
+            ctypes.c_uint64, ctypes.c_uint64, ctypes.c_float, ctypes.c_uint32,
+            ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
+            ctypes.c_void_p, ctypes.c_void_p,
+        ]
+        if cdll.tri_attn_version() != ABI_VERSION:
+            raise RuntimeError("libtrident_attn.so ABI version mismatch: rebuild it")
+        _lib = cdll
+    return _lib
+
+
+def check(status):
+    if status != 0:
+        raise RuntimeError("tri_attn: " + lib().tri_attn_strerror(status).decode())

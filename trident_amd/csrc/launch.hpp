@@ -1,0 +1,21 @@
+// Host-side launch entry points shared between the translation units of libtrident_attn.so.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "common.hpp"
+
+namespace tri {
+
+enum GenericKernel { kGenericFwd = 0, kGenericDelta = 1, kGenericDkdv = 2, kGenericDq = 3 };
+
+// generic.hip: any shape / dtype, vector-ALU fp32 arithmetic.
+int launch_generic_any(int which, int dtype, const KParams& p, hipStream_t stream);
+
+// mfma_*.hip: fp16/bf16, D in {64,128}, S a multiple of 128, 16-byte aligned rows.
+bool mfma_supported(int dtype, const KParams& p);
+int launch_mfma_fwd(int dtype, const KParams& p, hipStream_t stream);
+int launch_mfma_dq(int dtype, const KParams& p, hipStream_t stream);
+int launch_mfma_dkdv(int dtype, const KParams& p, hipStream_t stream);
+int launch_delta(int dtype, const KParams& p, hipStream_t stream);
+
+}  // namespace tri

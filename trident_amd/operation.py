@@ -1,0 +1,222 @@
+"""Attention autograd Function behind the reference's operator API.
+
+Mirrors trident/operation/attention.py:23-202: the same eight positional arguments, the same
+validation errors, the same saved state and the same 8-tuple returned by backward. The three
+Triton launches of the reference (attention.py:109, 161, 170) become calls into
+libtrident_attn.so (include/tri_attn.h).
+"""
+import ctypes
+from typing import Any
+
+import torch
+
+from . import _lib, config, util
+
+
+def _strides4(t: torch.Tensor):
+    s = list(t.stride())
+    if t.shape[-1] == 1:
+        s[-1] = 1
+    return s
+
+
+def _dense_rows(t: torch.Tensor) -> torch.Tensor:
+    """The kernels need unit stride along the last dimension and non-negative strides."""
+    if t.shape[-1] != 1 and t.stride(-1) != 1:
+        return t.contiguous()
+    return t
+
+
+def _next_seed():
+    fixed = config.dropout_seed
+    if fixed is None:
+        return int(torch.randint(0, 2**63 - 1, (1,), dtype=torch.int64).item()), 0
+    if isinstance(fixed, int):
+        fixed = (fixed, 0)
+    seed, offset = int(fixed[0]), int(fixed[1])
+    config.dropout_seed = (seed, offset + 1)
+    return seed, offset
+
+
+def _fill(args: _lib.TriAttnArgs, name: str, t: torch.Tensor, stride_field: str = None):
+    setattr(args, name, t.data_ptr())
+    if stride_field is not None:
+        getattr(args, stride_field)[:] = _strides4(t)
+
+
+def _base_args(query, mask, dropout_p, is_causal, softmax_scale, seed, offset):
+    args = _lib.TriAttnArgs()
+    args.struct_size = ctypes.sizeof(_lib.TriAttnArgs)
+    args.dtype = util.dtype(query.dtype)
+    args.B, args.H, args.S, args.D = query.shape
+    args.is_causal = 1 if is_causal else 0
+    args.softmax_scale = float(softmax_scale)
+    args.dropout_p = float(dropout_p)
+    args.seed = seed
+    args.offset = offset
+    if mask is not None:
+        args.mask_dtype = util.dtype(mask.dtype)
+        _fill(args, "mask", mask, "mask_stride")
+    args.stream = torch.cuda.current_stream(query.device).cuda_stream
+    return args
+
+
+def _expand_mask(mask: torch.Tensor, shape):
+    """View of the additive mask broadcast to [B,H,S,S] (stride 0 on broadcast dims)."""
+    view = mask
+    while view.dim() < 4:
+        view = view.unsqueeze(0)
+    view = view.expand(*shape)
+    if view.shape[-1] != 1 and view.stride(-1) != 1:
+        view = view.contiguous()
+    return view
+
+
+class Attention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx: Any, *args: Any, **kwargs: Any):
+        query, key, value, mask, dropout_p, is_causal, softmax_scale, use_accelerator = args
+
+        if query.dim() != 4 or key.dim() != 4 or value.dim() != 4:
+            raise ValueError("The dimension of query, key and value should be 4.")
+
+        if (
+            not util.is_pow2(query.shape[-2])
+            or not util.is_pow2(query.shape[-1])
+            or not util.is_pow2(key.shape[-2])
+            or not util.is_pow2(key.shape[-1])
+            or not util.is_pow2(value.shape[-2])
+            or not util.is_pow2(value.shape[-1])
+        ):
+            raise ValueError("Attention supports only for power of 2 size tensors.")
+
+        if mask is not None:
+            if is_causal:
+                raise ValueError("Error because both attn_mask and is_causal are set.")
+            if mask.dtype == torch.bool:
+                raise ValueError("Boolean mask is not supported yet.")
+
+        seed, offset = _next_seed() if dropout_p > 0.0 else (0, 0)
+
+        util.push_trace("Attention.__forward")
+        output, log_sum_exp = Attention._forward(
+            query, key, value, mask, dropout_p, is_causal, softmax_scale, seed, offset
+        )
+        util.pop_trace()
+
+        ctx.save_for_backward(query, key, value, output, log_sum_exp)
+        ctx.mask = mask
+        ctx.dropout_p = dropout_p
+        ctx.is_causal = is_causal
+        ctx.softmax_scale = softmax_scale
+        ctx.use_accelerator = use_accelerator
+        ctx.seed = seed
+        ctx.offset = offset
+
+        return output
+
+    @staticmethod
+    def backward(ctx: Any, *grad_outputs: Any):
+        (grad_output,) = grad_outputs
+        query, key, value, output, log_sum_exp = ctx.saved_tensors
+
+        util.push_trace("Attention.__backward")
+        grad_query, grad_key, grad_value, grad_mask = Attention._backward(
+            grad_output,
+            query,
+            key,
+            value,
+            output,
+            log_sum_exp,
+            ctx.mask,
+            ctx.softmax_scale,
+            ctx.dropout_p,
+            ctx.is_causal,
+            ctx.seed,
+            ctx.offset,
+            ctx.mask is not None and ctx.needs_input_grad[3],
+        )
+        util.pop_trace()
+
+        return grad_query, grad_key, grad_value, grad_mask, None, None, None, None
+
+    @staticmethod
+    def _forward(query, key, value, mask, dropout_p, is_causal, softmax_scale, seed, offset):
+        assert query.shape[-1] == key.shape[-1] and key.shape[-1] == value.shape[-1]
+        assert key.shape[-1] in {16, 32, 64, 128}
+        if not query.is_cuda:
+            raise RuntimeError("trident_amd attention runs on the GPU only; got a tensor on " + str(query.device))
+        if key.shape != query.shape or value.shape != query.shape:
+            raise ValueError("query, key and value must have the same shape.")
+        if key.dtype != query.dtype or value.dtype != query.dtype:
+            raise ValueError("query, key and value must have the same dtype.")
+
+        lib = _lib.lib()
+        query, key, value = _dense_rows(query), _dense_rows(key), _dense_rows(value)
+        num_batches, num_heads, y_size, x_size = query.shape
+        output = torch.empty(query.shape, device=query.device, dtype=query.dtype)
+        log2sum = torch.empty(num_batches, num_heads, y_size, device=query.device, dtype=torch.float32)
+        mask_view = _expand_mask(mask.detach(), (num_batches, num_heads, y_size, y_size)) if mask is not None else None
+
+        args = _base_args(query, mask_view, dropout_p, is_causal, softmax_scale, seed, offset)
+        _fill(args, "q", query, "q_stride")
+        _fill(args, "k", key, "k_stride")
+        _fill(args, "v", value, "v_stride")
+        _fill(args, "o", output, "o_stride")
+        _fill(args, "lse", log2sum)
+
+        util.push_trace("kernel.Attention.forward")
+        _lib.check(lib.tri_attn_fwd(ctypes.byref(args)))
+        util.pop_trace()
+
+        return output, log2sum
+
+    @staticmethod
+    def _backward(grad_output, query, key, value, output, log2sum, mask, softmax_scale, dropout_p, is_causal,
+                  seed, offset, want_grad_mask):
+        lib = _lib.lib()
+        query, key, value = _dense_rows(query), _dense_rows(key), _dense_rows(value)
+        grad_output = _dense_rows(grad_output)
+        num_batches, num_heads, y_size, x_size = output.shape
+        grad_query = torch.empty(query.shape, device=query.device, dtype=query.dtype)
+        grad_key = torch.empty(key.shape, device=key.device, dtype=key.dtype)
+        grad_value = torch.empty(value.shape, device=value.device, dtype=value.dtype)
+        delta = torch.empty_like(log2sum)
+        full = (num_batches, num_heads, y_size, y_size)
+        mask_view = _expand_mask(mask.detach(), full) if mask is not None else None
+        grad_mask_full = torch.empty(full, device=mask.device, dtype=mask.dtype) if want_grad_mask else None
+
+        args = _base_args(query, mask_view, dropout_p, is_causal, softmax_scale, seed, offset)
+        _fill(args, "q", query, "q_stride")
+        _fill(args, "k", key, "k_stride")
+        _fill(args, "v", value, "v_stride")
+        _fill(args, "o", output, "o_stride")
+        _fill(args, "lse", log2sum)
+        _fill(args, "d_o", grad_output, "do_stride")
+        _fill(args, "dq", grad_query, "dq_stride")
+        _fill(args, "dk", grad_key, "dk_stride")
+        _fill(args, "dv", grad_value, "dv_stride")
+        _fill(args, "delta", delta)
+        if grad_mask_full is not None:
+            _fill(args, "dmask", grad_mask_full, "dmask_stride")
+
+        util.push_trace("kernel.Softmax.backward_delta")
+        _lib.check(lib.tri_attn_bwd_delta(ctypes.byref(args)))
+        util.pop_trace()
+
+        util.push_trace("kernel.Attention.backward")
+        _lib.check(lib.tri_attn_bwd_dkdv(ctypes.byref(args)))
+        _lib.check(lib.tri_attn_bwd_dq(ctypes.byref(args)))
+        util.pop_trace()
+
+        grad_mask = None
+        if grad_mask_full is not None:
+            grad_mask = grad_mask_full
+            if tuple(mask.shape) != full:
+                # autograd semantics for a broadcast mask: sum over the broadcast dimensions
+                lead = 4 - mask.dim()
+                dims = [i for i in range(4) if i < lead or mask.shape[i - lead] != full[i]]
+                grad_mask = grad_mask_full.float().sum(dim=dims, keepdim=True).to(mask.dtype)
+                grad_mask = grad_mask.reshape(mask.shape)
+
+        return grad_query, grad_key, grad_value, grad_mask
