@@ -96,9 +96,11 @@ def attention_forward(q, k, v, mask=None, dropout_p=0.0, is_causal=False, scale=
 
 
 def attention_backward(q, k, v, d_out, mask=None, dropout_p=0.0, is_causal=False, scale=None, seed=0, offset=0,
-                       want_dmask=False):
+                       want_dmask=False, o=None):
     """Closed-form gradients. Returns (dQ, dK, dV, dMask or None, delta [B,H,S]).
-    dMask has the mask's own (possibly broadcast) shape: summed over broadcast dims."""
+    dMask has the mask's own (possibly broadcast) shape: summed over broadcast dims.
+    ``o``: the saved forward output the backward is handed (the reference computes delta from the
+    stored output tensor, trident/operation/attention.py:139-164); None recomputes it exactly."""
     q = np.asarray(q, dtype=np.float64)
     k = np.asarray(k, dtype=np.float64)
     v = np.asarray(v, dtype=np.float64)
@@ -117,8 +119,8 @@ def attention_backward(q, k, v, d_out, mask=None, dropout_p=0.0, is_causal=False
             p, _ = _softmax_rows(s)
             z = _keep_scale(seed, offset, b * H + h, S, dropout_p)
             pz = p if z is None else p * z
-            o = pz @ v[b, h]
-            dlt = np.sum(d_out[b, h] * o, axis=-1)
+            o_bh = pz @ v[b, h] if o is None else np.asarray(o[b, h], dtype=np.float64)
+            dlt = np.sum(d_out[b, h] * o_bh, axis=-1)
             dp = d_out[b, h] @ v[b, h].T
             if z is not None:
                 dp = dp * z

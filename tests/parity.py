@@ -41,6 +41,8 @@ def oracle_forward(q, k, v, mask=None, dropout_p=0.0, is_causal=False, scale=Non
 
 
 def oracle_backward(q, k, v, d_o, mask=None, dropout_p=0.0, is_causal=False, scale=None, seed=0, offset=0,
-                    want_dmask=False):
+                    want_dmask=False, o=None):
+    """``o``: the forward output the backward under test was handed (already checked against the
+    oracle's forward); delta is defined on that stored tensor."""
     return oracle.attention_backward(to64(q), to64(k), to64(v), to64(d_o), to64(mask), dropout_p, is_causal, scale,
-                                     seed, offset, want_dmask)
+                                     seed, offset, want_dmask, o=to64(o))

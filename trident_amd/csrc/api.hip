@@ -146,7 +146,7 @@ int tri_attn_fwd(const TriAttnArgs* args) {
     int rc = make_params(args, 1, &p);
     if (rc) return rc;
     hipStream_t st = static_cast<hipStream_t>(args->stream);
-    if (mfma_supported(args->dtype, p)) return launch_mfma_fwd(args->dtype, p, st);
+    if (mfma_supported(kMfmaFwd, args->dtype, p)) return launch_mfma_fwd(args->dtype, p, st);
     return launch_generic_any(kGenericFwd, args->dtype, p, st);
 }
 
@@ -162,7 +162,7 @@ int tri_attn_bwd_dkdv(const TriAttnArgs* args) {
     int rc = make_params(args, 4, &p);
     if (rc) return rc;
     hipStream_t st = static_cast<hipStream_t>(args->stream);
-    if (mfma_supported(args->dtype, p)) return launch_mfma_dkdv(args->dtype, p, st);
+    if (mfma_supported(kMfmaDkdv, args->dtype, p)) return launch_mfma_dkdv(args->dtype, p, st);
     return launch_generic_any(kGenericDkdv, args->dtype, p, st);
 }
 
@@ -171,7 +171,7 @@ int tri_attn_bwd_dq(const TriAttnArgs* args) {
     int rc = make_params(args, 8, &p);
     if (rc) return rc;
     hipStream_t st = static_cast<hipStream_t>(args->stream);
-    if (mfma_supported(args->dtype, p) && p.dmask == nullptr) return launch_mfma_dq(args->dtype, p, st);
+    if (mfma_supported(kMfmaDq, args->dtype, p)) return launch_mfma_dq(args->dtype, p, st);
     return launch_generic_any(kGenericDq, args->dtype, p, st);
 }
 

@@ -96,7 +96,8 @@ __device__ __forceinline__ Philox4 dropout_block(const KParams& p, uint32_t bh, 
 }
 __device__ __forceinline__ bool dropout_keep(const KParams& p, uint32_t bh, uint32_t i, uint32_t j) {
     const Philox4 r = dropout_block(p, bh, i >> 2, j >> 2);
-    const uint32_t word = r.w[i & 3];
+    const uint32_t s = i & 3;
+    const uint32_t word = s == 0 ? r.w[0] : (s == 1 ? r.w[1] : (s == 2 ? r.w[2] : r.w[3]));
     const int u8 = static_cast<int>((word >> (8 * (j & 3))) & 0xffu);
     return u8 >= p.thr8;
 }

@@ -12,7 +12,8 @@ enum GenericKernel { kGenericFwd = 0, kGenericDelta = 1, kGenericDkdv = 2, kGene
 int launch_generic_any(int which, int dtype, const KParams& p, hipStream_t stream);
 
 // mfma_*.hip: fp16/bf16, D in {64,128}, S a multiple of 128, 16-byte aligned rows.
-bool mfma_supported(int dtype, const KParams& p);
+enum MfmaKernel { kMfmaFwd = 0, kMfmaDkdv = 1, kMfmaDq = 2 };
+bool mfma_supported(int which, int dtype, const KParams& p);
 int launch_mfma_fwd(int dtype, const KParams& p, hipStream_t stream);
 int launch_mfma_dq(int dtype, const KParams& p, hipStream_t stream);
 int launch_mfma_dkdv(int dtype, const KParams& p, hipStream_t stream);

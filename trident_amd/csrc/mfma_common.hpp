@@ -1,0 +1,209 @@
+// Building blocks of the matrix-core (MFMA) attention kernels for gfx950.
+//
+// All three kernels (forward, dQ, dK/dV) use v_mfma_f32_32x32x16_{bf16,f16}:
+//   A is 32(M) x 16(K): lane l holds row M = l % 32 and the 8 K-slots 8*(l/32) .. 8*(l/32)+7
+//   B is 16(K) x 32(N): lane l holds column N = l % 32 and the same 8 K-slots
+//   C/D is 32 x 32 fp32: lane l holds column N = l % 32 and, in register i (0..15),
+//   row M = 8*(i/4) + 4*(l/32) + i%4.
+// The kernels are written "transposed" (S^T = K Q^T, O^T = V^T P^T, ...) so that the lane
+// index is always the row the softmax statistics belong to: row maxima, sums, the LSE and
+// delta are per-lane scalars, and a C tile can be fed back as the B operand of the next
+// MFMA without leaving registers: registers 8g .. 8g+7 of a C tile, converted to 16 bit,
+// are the 8 K-slots of K-step g; slot t of lane-half h then stands for tile row
+// 16g + 8*(t/4) + 4h + t%4, and the A operand of that MFMA is stored in LDS in exactly
+// that slot order ("slot-permuted" transposed tiles below).
+#pragma once
+#include "common.hpp"
+
+namespace tri {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef bf16_t bf16x8 __attribute__((ext_vector_type(8)));
+typedef f16_t f16x8 __attribute__((ext_vector_type(8)));
+typedef bf16_t bf16x2 __attribute__((ext_vector_type(2)));
+typedef f16_t f16x2 __attribute__((ext_vector_type(2)));
+
+template <typename T>
+struct Mma;
+template <>
+struct Mma<bf16_t> {
+    static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                       0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+        bf16x2 v = {static_cast<bf16_t>(lo), static_cast<bf16_t>(hi)};
+        return __builtin_bit_cast(uint32_t, v);
+    }
+    static __device__ __forceinline__ float lo(uint32_t w) { return __uint_as_float(w << 16); }
+    static __device__ __forceinline__ float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+};
+template <>
+struct Mma<f16_t> {
+    static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
+                                                      0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+        f16x2 v = {static_cast<f16_t>(lo), static_cast<f16_t>(hi)};
+        return __builtin_bit_cast(uint32_t, v);
+    }
+    static __device__ __forceinline__ float lo(uint32_t w) {
+        return static_cast<float>(__builtin_bit_cast(f16x2, w)[0]);
+    }
+    static __device__ __forceinline__ float hi(uint32_t w) {
+        return static_cast<float>(__builtin_bit_cast(f16x2, w)[1]);
+    }
+};
+
+// 8 consecutive C registers -> one B operand (8 K-slots) in the 16-bit type.
+template <typename T>
+__device__ __forceinline__ u32x4 pack8(const float* x) {
+    u32x4 r;
+    r.x = Mma<T>::pack2(x[0], x[1]);
+    r.y = Mma<T>::pack2(x[2], x[3]);
+    r.z = Mma<T>::pack2(x[4], x[5]);
+    r.w = Mma<T>::pack2(x[6], x[7]);
+    return r;
+}
+
+__device__ __forceinline__ f32x16 zero16() {
+    f32x16 z;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) z[i] = 0.f;
+    return z;
+}
+
+// Row index inside a 32-row C tile of register i for lane-half h.
+__device__ __forceinline__ int c_row(int i, int h) { return 8 * (i >> 2) + 4 * h + (i & 3); }
+
+__device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32); }
+
+// ---------------------------------------------------------------- LDS tiles
+// Row-major tile [ROWS][D] of 16-bit elements, rows padded by 16 bytes so that the 32 lanes
+// of an A-operand read (32 consecutive rows, same 16-byte column chunk) hit distinct banks.
+template <int D>
+struct RowTile {
+    static constexpr int kStride = D * 2 + 16;  // bytes
+    static constexpr int bytes(int rows) { return rows * kStride; }
+    // 16-byte chunk c of row r
+    static __device__ __forceinline__ int off(int r, int c) { return r * kStride + c * 16; }
+};
+
+// Transposed, slot-permuted tile of a [64][D] source: LDS row d (128 bytes) holds the 64
+// source rows of column d; source row r sits at slot 16*(r/16) + 8*((r/4)%2) + 4*((r/8)%2) + r%4,
+// and 16-byte chunks are XOR-swizzled with (d%8)^((d/8)%8) so that both the 8-byte writes
+// (16 lanes = 16 different d, stride 8) and the 16-byte A-operand reads (32 consecutive d) are
+// bank-conflict free.
+struct TransTile {
+    static constexpr int kRowBytes = 128;
+    static constexpr int bytes(int d) { return d * kRowBytes; }
+    static __device__ __forceinline__ int swz(int d) { return (d & 7) ^ ((d >> 3) & 7); }
+    // A operand: LDS row d, K-step ks (16 source rows), lane-half h
+    static __device__ __forceinline__ int read_off(int d, int ks, int h) {
+        return d * kRowBytes + (((2 * ks + h) ^ swz(d)) << 4);
+    }
+    // 8-byte write of source rows 4*rq .. 4*rq+3 (rq = 0..15) of column d
+    static __device__ __forceinline__ int write_off(int d, int rq) {
+        const int chunk = 2 * (rq >> 2) + (rq & 1);
+        return d * kRowBytes + ((chunk ^ swz(d)) << 4) + ((rq >> 1) & 1) * 8;
+    }
+};
+
+__device__ __forceinline__ u32x4 lds_read16(const char* smem, int off) {
+    return *reinterpret_cast<const u32x4*>(smem + off);
+}
+__device__ __forceinline__ void lds_write16(char* smem, int off, u32x4 v) { *reinterpret_cast<u32x4*>(smem + off) = v; }
+__device__ __forceinline__ void lds_write8(char* smem, int off, u32x2 v) { *reinterpret_cast<u32x2*>(smem + off) = v; }
+
+// Global -> registers -> LDS staging of one [64][D] tile by 256 threads, row-major target.
+template <int D>
+struct RowStage {
+    static constexpr int kChunksPerRow = D / 8;
+    static constexpr int kPerThread = 64 * kChunksPerRow / 256;  // 4 for D=128, 2 for D=64
+    u32x4 r[kPerThread];
+    __device__ __forceinline__ void load(const char* base, int64_t row_stride_bytes, int tid) {
+#pragma unroll
+        for (int i = 0; i < kPerThread; ++i) {
+            const int g = tid + 256 * i;
+            const int row = g / kChunksPerRow, c = g % kChunksPerRow;
+            r[i] = *reinterpret_cast<const u32x4*>(base + row * row_stride_bytes + c * 16);
+        }
+    }
+    __device__ __forceinline__ void store(char* smem, int tid) const {
+#pragma unroll
+        for (int i = 0; i < kPerThread; ++i) {
+            const int g = tid + 256 * i;
+            const int row = g / kChunksPerRow, c = g % kChunksPerRow;
+            lds_write16(smem, RowTile<D>::off(row, c), r[i]);
+        }
+    }
+};
+
+// Global -> registers -> LDS staging of one [64][D] tile into a TransTile: thread (rq, c) holds
+// source rows 4rq..4rq+3, columns c*D/16 .. (c+1)*D/16-1 (16 lanes cover one source row, so
+// the global loads stay row-contiguous).
+template <typename T, int D>
+struct TransStage {
+    static constexpr int kCols = D / 16;      // 8 for D=128 (16-byte loads), 4 for D=64 (8-byte loads)
+    static constexpr int kWords = kCols / 2;
+    uint32_t r[4][kWords];
+    __device__ __forceinline__ void load(const char* base, int64_t row_stride_bytes, int tid) {
+        const int rq = tid >> 4, c = tid & 15;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            const char* src = base + (4 * rq + a) * row_stride_bytes + c * kCols * 2;
+            if constexpr (kWords == 4) {
+                const u32x4 v = *reinterpret_cast<const u32x4*>(src);
+                r[a][0] = v.x; r[a][1] = v.y; r[a][2] = v.z; r[a][3] = v.w;
+            } else {
+                const u32x2 v = *reinterpret_cast<const u32x2*>(src);
+                r[a][0] = v.x; r[a][1] = v.y;
+            }
+        }
+    }
+    __device__ __forceinline__ void store(char* smem, int tid) const {
+        const int rq = tid >> 4, c = tid & 15;
+#pragma unroll
+        for (int wd = 0; wd < kWords; ++wd) {
+            // even column: low halves of the four rows; odd column: high halves
+            u32x2 ev, od;
+            ev.x = __builtin_amdgcn_perm(r[1][wd], r[0][wd], 0x05040100u);
+            ev.y = __builtin_amdgcn_perm(r[3][wd], r[2][wd], 0x05040100u);
+            od.x = __builtin_amdgcn_perm(r[1][wd], r[0][wd], 0x07060302u);
+            od.y = __builtin_amdgcn_perm(r[3][wd], r[2][wd], 0x07060302u);
+            const int d = c * kCols + 2 * wd;
+            lds_write8(smem, TransTile::write_off(d, rq), ev);
+            lds_write8(smem, TransTile::write_off(d + 1, rq), od);
+        }
+    }
+};
+
+// Workgroup -> (head, tile) mapping. Workgroups are dealt round-robin to the 8 XCDs, each with
+// its own L2: give every XCD whole heads, walk the tiles of a head consecutively so its K/V
+// stay in that L2, and start with the heaviest tiles (highest index first when `reverse`).
+__device__ __forceinline__ void map_block(int bid, int num_heads, int num_tiles, bool reverse, int* bh, int* tile) {
+    int head, t;
+    if ((num_heads & 7) == 0) {
+        const int xcd = bid & 7, slot = bid >> 3;
+        head = (slot / num_tiles) * 8 + xcd;
+        t = slot % num_tiles;
+    } else {
+        head = bid / num_tiles;
+        t = bid % num_tiles;
+    }
+    *bh = head;
+    *tile = reverse ? num_tiles - 1 - t : t;
+}
+
+// Dropout bytes for 4 consecutive columns j0..j0+3 (j0 % 4 == 0) of row i: one 32-bit word.
+__device__ __forceinline__ uint32_t dropout_word(const KParams& p, uint32_t bh, uint32_t i, uint32_t j0) {
+    const Philox4 r = dropout_block(p, bh, i >> 2, j0 >> 2);
+    const uint32_t s = i & 3;
+    return s == 0 ? r.w[0] : (s == 1 ? r.w[1] : (s == 2 ? r.w[2] : r.w[3]));
+}
+
+}  // namespace tri

@@ -1,0 +1,210 @@
+// Forward attention on the matrix cores: online-softmax flash kernel for fp16/bf16,
+// D in {64,128}, S a multiple of 128 (replaces trident/kernel/attention.py:33-165).
+//
+// One workgroup (4 waves) owns 128 query rows, one wave 32 of them. Q stays in registers as
+// the B operand of S^T = K Q^T; K (row-major, padded) and V^T (transposed, slot-permuted)
+// tiles of 64 keys are double-buffered in LDS and filled with 16-byte global loads issued one
+// tile ahead. S^T and O^T = V^T P^T accumulate in fp32; P goes from the S^T accumulators to
+// the B operand of the second MFMA in registers. The row statistics live one per lane; the
+// two lane halves of a row are combined with one cross-lane exchange per tile.
+#include "launch.hpp"
+#include "mfma_common.hpp"
+
+namespace tri {
+namespace {
+
+constexpr int kBM = 128;  // query rows per workgroup
+constexpr int kBN = 64;   // keys per tile
+
+enum MaskKind { kNoMask = 0, kMaskF32 = 1, kMaskT = 2 };
+
+template <typename T, int D, bool CAUSAL, int MASK, bool DROPOUT>
+__global__ __launch_bounds__(256, 2) void mfma_fwd_kernel(const KParams p) {
+    constexpr int kKBytes = RowTile<D>::bytes(kBN);
+    constexpr int kVBytes = TransTile::bytes(D);
+    constexpr int kStageBytes = kKBytes + kVBytes;
+    constexpr int KK = D / 16;  // K-steps of S^T
+    constexpr int DB = D / 32;  // 32-row blocks of O^T
+    __shared__ __attribute__((aligned(16))) char smem[2 * kStageBytes];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+    int bh, qt;
+    map_block(blockIdx.x, p.B * p.H, p.S / kBM, true, &bh, &qt);
+    const int b = bh / p.H, hd = bh % p.H;
+    const int q0 = qt * kBM;
+    const int wrow0 = q0 + 32 * wave;  // first query row of this wave
+    const int qrow = wrow0 + l32;
+
+    const char* qbase = static_cast<const char*>(p.q) + (b * p.qs[0] + hd * p.qs[1]) * 2;
+    const char* kbase = static_cast<const char*>(p.k) + (b * p.ks[0] + hd * p.ks[1]) * 2;
+    const char* vbase = static_cast<const char*>(p.v) + (b * p.vs[0] + hd * p.vs[1]) * 2;
+    const int64_t krow_bytes = p.ks[2] * 2, vrow_bytes = p.vs[2] * 2;
+
+    u32x4 qf[KK];
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk)
+        qf[kk] = *reinterpret_cast<const u32x4*>(qbase + qrow * p.qs[2] * 2 + (2 * kk + h) * 16);
+
+    f32x16 oacc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) oacc[db] = zero16();
+    float m = -INFINITY, l = 0.f;  // running max (log2 domain, scaled) and this lane's partial sum
+
+    const int n_tiles = CAUSAL ? (q0 + kBM) / kBN : p.S / kBN;
+    const float c = p.scale_log2;
+
+    RowStage<D> kst;
+    TransStage<T, D> vst;
+    kst.load(kbase, krow_bytes, tid);
+    vst.load(vbase, vrow_bytes, tid);
+    kst.store(smem, tid);
+    vst.store(smem + kKBytes, tid);
+    __syncthreads();
+
+    for (int j = 0; j < n_tiles; ++j) {
+        const char* sK = smem + (j & 1) * kStageBytes;
+        const char* sV = sK + kKBytes;
+        const int t0 = j * kBN;
+        const bool more = j + 1 < n_tiles;
+        if (more) {
+            kst.load(kbase + (t0 + kBN) * krow_bytes, krow_bytes, tid);
+            vst.load(vbase + (t0 + kBN) * vrow_bytes, vrow_bytes, tid);
+        }
+        const bool active = !CAUSAL || t0 <= wrow0 + 31;
+        if (active) {
+            float x[32];  // scores of this lane: x[16*kb + i] is key t0 + 32*kb + c_row(i,h)
+            // additive mask for this lane's row: issued before the MFMAs, used after them
+            float mk[MASK != kNoMask ? 32 : 1];
+            if constexpr (MASK != kNoMask) {
+                const int64_t mrow = b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(qrow) * p.ms[2] + t0;
+#pragma unroll
+                for (int g = 0; g < 8; ++g) {
+                    const int key0 = 32 * (g >> 2) + 8 * (g & 3) + 4 * h;
+                    if constexpr (MASK == kMaskF32) {
+                        const f32x4 v = *reinterpret_cast<const f32x4*>(static_cast<const float*>(p.mask) + mrow + key0);
+                        mk[4 * g + 0] = v.x; mk[4 * g + 1] = v.y; mk[4 * g + 2] = v.z; mk[4 * g + 3] = v.w;
+                    } else {
+                        const u32x2 v = *reinterpret_cast<const u32x2*>(static_cast<const T*>(p.mask) + mrow + key0);
+                        mk[4 * g + 0] = Mma<T>::lo(v.x); mk[4 * g + 1] = Mma<T>::hi(v.x);
+                        mk[4 * g + 2] = Mma<T>::lo(v.y); mk[4 * g + 3] = Mma<T>::hi(v.y);
+                    }
+                }
+            }
+            // S^T = K Q^T
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                f32x16 st = zero16();
+#pragma unroll
+                for (int kk = 0; kk < KK; ++kk) {
+                    const u32x4 a = lds_read16(sK, RowTile<D>::off(32 * kb + l32, 2 * kk + h));
+                    st = Mma<T>::run(a, qf[kk], st);
+                }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) x[16 * kb + i] = st[i];
+            }
+            // scores in the log2 domain; without a mask the scale is folded into the exponent
+            if constexpr (MASK != kNoMask) {
+#pragma unroll
+                for (int e = 0; e < 32; ++e) x[e] = fmaf(mk[e], kLog2e, x[e] * c);
+            }
+            if (CAUSAL && t0 + kBN - 1 > wrow0) {
+#pragma unroll
+                for (int e = 0; e < 32; ++e) {
+                    const int key = t0 + 32 * (e >> 4) + c_row(e & 15, h);
+                    x[e] = key <= qrow ? x[e] : -INFINITY;
+                }
+            }
+            float mx = x[0];
+#pragma unroll
+            for (int e = 1; e < 32; ++e) mx = fmaxf(mx, x[e]);
+            mx = fmaxf(mx, xor32(mx));
+            if constexpr (MASK == kNoMask) mx *= c;
+            const float m_new = fmaxf(m, mx);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            const float alpha = fast_exp2(m - m_use);
+            float psum = 0.f;
+#pragma unroll
+            for (int e = 0; e < 32; ++e) {
+                if constexpr (MASK == kNoMask) x[e] = fast_exp2(fmaf(x[e], c, -m_use));
+                else x[e] = fast_exp2(x[e] - m_use);
+                psum += x[e];
+            }
+            l = fmaf(l, alpha, psum);
+            m = m_new;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) oacc[db][i] *= alpha;
+            if constexpr (DROPOUT) {
+#pragma unroll
+                for (int g = 0; g < 8; ++g) {
+                    const int key0 = t0 + 32 * (g >> 2) + 8 * (g & 3) + 4 * h;
+                    const uint32_t w = dropout_word(p, bh, qrow, key0);
+#pragma unroll
+                    for (int bb = 0; bb < 4; ++bb) {
+                        const bool keep = static_cast<int>((w >> (8 * bb)) & 0xffu) >= p.thr8;
+                        x[4 * g + bb] = keep ? x[4 * g + bb] * p.zscale : 0.f;
+                    }
+                }
+            }
+            // O^T += V^T P^T
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                const u32x4 pb = pack8<T>(&x[8 * ks]);
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    const u32x4 a = lds_read16(sV, TransTile::read_off(32 * db + l32, ks, h));
+                    oacc[db] = Mma<T>::run(a, pb, oacc[db]);
+                }
+            }
+        }
+        if (more) {
+            char* nK = smem + ((j + 1) & 1) * kStageBytes;
+            kst.store(nK, tid);
+            vst.store(nK + kKBytes, tid);
+        }
+        __syncthreads();
+    }
+
+    l += xor32(l);
+    const float inv = 1.f / l;
+    char* orow = static_cast<char*>(p.o) + (b * p.os[0] + hd * p.os[1] + static_cast<int64_t>(qrow) * p.os[2]) * 2;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            u32x2 v;
+            v.x = Mma<T>::pack2(oacc[db][4 * g + 0] * inv, oacc[db][4 * g + 1] * inv);
+            v.y = Mma<T>::pack2(oacc[db][4 * g + 2] * inv, oacc[db][4 * g + 3] * inv);
+            *reinterpret_cast<u32x2*>(orow + (32 * db + 8 * g + 4 * h) * 2) = v;
+        }
+    if (h == 0) p.lse[static_cast<int64_t>(bh) * p.S + qrow] = m + fast_log2(l);
+}
+
+template <typename T, int D, bool CAUSAL, int MASK>
+int launch_fwd_dropout(const KParams& p, hipStream_t stream) {
+    const dim3 grid(p.B * p.H * (p.S / kBM)), block(256);
+    if (p.thr8 > 0) hipLaunchKernelGGL((mfma_fwd_kernel<T, D, CAUSAL, MASK, true>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((mfma_fwd_kernel<T, D, CAUSAL, MASK, false>), grid, block, 0, stream, p);
+    return static_cast<int>(hipGetLastError());
+}
+
+template <typename T, int D>
+int launch_fwd_variant(int dtype, const KParams& p, hipStream_t stream) {
+    if (p.causal) return launch_fwd_dropout<T, D, true, kNoMask>(p, stream);
+    if (p.mask == nullptr) return launch_fwd_dropout<T, D, false, kNoMask>(p, stream);
+    if (p.mask_dtype == TRI_ATTN_F32) return launch_fwd_dropout<T, D, false, kMaskF32>(p, stream);
+    if (p.mask_dtype == dtype) return launch_fwd_dropout<T, D, false, kMaskT>(p, stream);
+    return TRI_ATTN_EDTYPE;
+}
+
+}  // namespace
+
+int launch_mfma_fwd(int dtype, const KParams& p, hipStream_t stream) {
+    if (dtype == TRI_ATTN_BF16)
+        return p.D == 128 ? launch_fwd_variant<bf16_t, 128>(dtype, p, stream) : launch_fwd_variant<bf16_t, 64>(dtype, p, stream);
+    return p.D == 128 ? launch_fwd_variant<f16_t, 128>(dtype, p, stream) : launch_fwd_variant<f16_t, 64>(dtype, p, stream);
+}
+
+}  // namespace tri

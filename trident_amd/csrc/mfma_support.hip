@@ -1,0 +1,86 @@
+// Which calls the matrix-core kernels take, and the delta pre-pass.
+#include "launch.hpp"
+#include "mfma_common.hpp"
+
+namespace tri {
+namespace {
+
+bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
+bool strides8(const int64_t* s) { return (s[0] % 8) == 0 && (s[1] % 8) == 0 && (s[2] % 8) == 0; }
+
+// delta[bh, i] = sum_d dO[i,d] * O[i,d] (trident/kernel/softmax.py:184-238 as attention uses it).
+// Pure streaming: 16-byte loads, D/8 lanes per row, fp32 accumulation, one fp32 store per row.
+template <typename T, int D>
+__global__ __launch_bounds__(256) void delta_kernel(const KParams p) {
+    constexpr int kLanes = D / 8;           // lanes per row: 16 (D=128) or 8 (D=64)
+    constexpr int kRowsPerBlock = 256 / kLanes;
+    const int sub = threadIdx.x % kLanes;
+    const int64_t row_lin = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + threadIdx.x / kLanes;
+    const int64_t total = static_cast<int64_t>(p.B) * p.H * p.S;
+    if (row_lin >= total) return;  // whole lane groups leave together: total is a multiple of 128
+    const int row = static_cast<int>(row_lin % p.S);
+    const int bh = static_cast<int>(row_lin / p.S);
+    const int b = bh / p.H, h = bh % p.H;
+    const T* orow = static_cast<const T*>(p.o) + b * p.os[0] + h * p.os[1] + static_cast<int64_t>(row) * p.os[2];
+    const T* grow = static_cast<const T*>(p.d_o) + b * p.dos[0] + h * p.dos[1] + static_cast<int64_t>(row) * p.dos[2];
+    const u32x4 ov = *reinterpret_cast<const u32x4*>(orow + sub * 8);
+    const u32x4 gv = *reinterpret_cast<const u32x4*>(grow + sub * 8);
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        acc = fmaf(Mma<T>::lo(ov[i]), Mma<T>::lo(gv[i]), acc);
+        acc = fmaf(Mma<T>::hi(ov[i]), Mma<T>::hi(gv[i]), acc);
+    }
+#pragma unroll
+    for (int s = 1; s < kLanes; s <<= 1) acc += __shfl_xor(acc, s);
+    if (sub == 0) p.delta[row_lin] = acc;
+}
+
+template <typename T, int D>
+int launch_delta_t(const KParams& p, hipStream_t stream) {
+    constexpr int kRowsPerBlock = 256 / (D / 8);
+    const int64_t total = static_cast<int64_t>(p.B) * p.H * p.S;
+    hipLaunchKernelGGL((delta_kernel<T, D>), dim3(static_cast<unsigned>((total + kRowsPerBlock - 1) / kRowsPerBlock)),
+                       dim3(256), 0, stream, p);
+    return static_cast<int>(hipGetLastError());
+}
+
+}  // namespace
+
+bool mfma_supported(int which, int dtype, const KParams& p) {
+    if (dtype != TRI_ATTN_F16 && dtype != TRI_ATTN_BF16) return false;
+    if (p.D != 64 && p.D != 128) return false;
+    if (p.S % 128 != 0) return false;
+    if (!(p.scale > 0.f)) return false;  // the kernels take row maxima before scaling
+    if (!aligned16(p.q) || !aligned16(p.k) || !aligned16(p.v)) return false;
+    if (!strides8(p.qs) || !strides8(p.ks) || !strides8(p.vs)) return false;
+    if (p.mask != nullptr) {
+        if (p.mask_dtype != TRI_ATTN_F32 && p.mask_dtype != dtype) return false;
+        if (!aligned16(p.mask)) return false;
+        if ((p.ms[0] % 4) || (p.ms[1] % 4) || (p.ms[2] % 4)) return false;
+    }
+    switch (which) {
+        case kMfmaFwd:
+            return aligned16(p.o) && strides8(p.os);
+        case kMfmaDkdv:
+        case kMfmaDq:
+            return false;
+        default:
+            return false;
+    }
+}
+
+int launch_mfma_dq(int, const KParams&, hipStream_t) { return TRI_ATTN_ESHAPE; }
+int launch_mfma_dkdv(int, const KParams&, hipStream_t) { return TRI_ATTN_ESHAPE; }
+
+int launch_delta(int dtype, const KParams& p, hipStream_t stream) {
+    const bool vec = (dtype == TRI_ATTN_F16 || dtype == TRI_ATTN_BF16) && (p.D == 64 || p.D == 128) &&
+                     aligned16(p.o) && aligned16(p.d_o) && strides8(p.os) && strides8(p.dos) &&
+                     (static_cast<int64_t>(p.B) * p.H * p.S) % 128 == 0;
+    if (!vec) return launch_generic_any(kGenericDelta, dtype, p, stream);
+    if (dtype == TRI_ATTN_BF16)
+        return p.D == 128 ? launch_delta_t<bf16_t, 128>(p, stream) : launch_delta_t<bf16_t, 64>(p, stream);
+    return p.D == 128 ? launch_delta_t<f16_t, 128>(p, stream) : launch_delta_t<f16_t, 64>(p, stream);
+}
+
+}  // namespace tri
