@@ -1,0 +1,248 @@
+#!/usr/bin/env python3
+"""Attention hot-path benchmark on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--report]
+
+A step is one pass of the hot path over one batch of synthetic input: forward, then the
+backward pre-pass (delta), dK/dV and dQ, called through the C ABI on tensors that are already
+resident in HBM. The default workload is C3 (bf16, causal, B=2 H=16 S=4096 D=128), the one the
+headline metric is quoted on. Rank 0 prints ONE JSON line on stdout; --report additionally
+prints forward and forward+backward figures for all five configurations on stderr.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"bf16": 2516.6, "fp16": 2516.6, "fp32": 157.3}  # MI355X dense MFMA peaks (256 CU x 2.4 GHz)
+HBM_PEAK_GBS = 8000.0
+
+# HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (see profiles/); None where not measured.
+MEASURED_TRAFFIC = {}
+
+
+def _dtype_name(dtype):
+    import torch
+
+    return {torch.float32: "fp32", torch.float16: "fp16", torch.bfloat16: "bf16"}[dtype]
+
+
+class Path:
+    """The four C-ABI calls of one step on preallocated device tensors."""
+
+    def __init__(self, w, dev):
+        import torch
+
+        from trident_amd import _lib, operation, workloads
+
+        self.w = w
+        self.lib = _lib.lib()
+        self.check = _lib.check
+        q, k, v, d_o, mask = workloads.make_inputs(w)
+        self.q, self.k, self.v, self.d_o = [x.to(dev) for x in (q, k, v, d_o)]
+        self.mask = None if mask is None else mask.to(dev)
+        B, H, S, D = self.q.shape
+        self.o = torch.empty_like(self.q)
+        self.lse = torch.empty(B, H, S, device=dev, dtype=torch.float32)
+        self.delta = torch.empty_like(self.lse)
+        self.dq, self.dk, self.dv = [torch.empty_like(self.q) for _ in range(3)]
+        mview = operation._expand_mask(self.mask, (B, H, S, S)) if self.mask is not None else None
+        self.mview = mview
+        args = operation._base_args(self.q, mview, w.dropout_p, w.is_causal, w.scale, w.dropout_seed, 0)
+        for name, t, field in [("q", self.q, "q_stride"), ("k", self.k, "k_stride"), ("v", self.v, "v_stride"),
+                               ("o", self.o, "o_stride"), ("d_o", self.d_o, "do_stride"), ("dq", self.dq, "dq_stride"),
+                               ("dk", self.dk, "dk_stride"), ("dv", self.dv, "dv_stride")]:
+            operation._fill(args, name, t, field)
+        operation._fill(args, "lse", self.lse)
+        operation._fill(args, "delta", self.delta)
+        self.args = args
+        ref = ctypes.byref(args)
+        self.kernels = [("fwd", lambda: self.check(self.lib.tri_attn_fwd(ref)))]
+        if w.backward:
+            self.kernels += [
+                ("bwd_delta", lambda: self.check(self.lib.tri_attn_bwd_delta(ref))),
+                ("bwd_dkdv", lambda: self.check(self.lib.tri_attn_bwd_dkdv(ref))),
+                ("bwd_dq", lambda: self.check(self.lib.tri_attn_bwd_dq(ref))),
+            ]
+
+    def algorithmic_flops(self, kernel):
+        """Flops credited per launch: forward 4 B H S^2 D; of the 10 B H S^2 D of the backward,
+        dK/dV is credited its four GEMMs (S, dP, dV, dK) and dQ one (dQ); the S and dP that the
+        dQ pass recomputes are not credited. Causal halves everything."""
+        unit = self.w.flops() / 4.0  # 1 * B H S^2 D (x 1/2 causal)
+        return {"fwd": 4.0, "bwd_dkdv": 8.0, "bwd_dq": 2.0, "bwd_delta": 0.0}[kernel] * unit
+
+    def algorithmic_bytes(self, kernel):
+        B, H, S, D = self.q.shape
+        elt = self.q.element_size()
+        if kernel == "bwd_delta":
+            return 2 * B * H * S * D * elt + 4 * B * H * S
+        return None
+
+
+def run_steps(path, steps, warmup):
+    """Returns (ms per step by wall clock, {kernel: avg ms} from HIP events on the launch stream)."""
+    import torch
+
+    for _ in range(warmup):
+        for _, fn in path.kernels:
+            fn()
+    torch.cuda.synchronize()
+    n = len(path.kernels)
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(n + 1)] for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for s in range(steps):
+        events[s][0].record()
+        for i, (_, fn) in enumerate(path.kernels):
+            fn()
+            events[s][i + 1].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    per_kernel = {}
+    for i, (name, _) in enumerate(path.kernels):
+        per_kernel[name] = sum(events[s][i].elapsed_time(events[s][i + 1]) for s in range(steps)) / steps
+    return wall_ms, per_kernel
+
+
+def cpu_baseline(w, reps=3):
+    """torch.nn.functional.scaled_dot_product_attention on the host cores (the op the reference's
+    tests take as their oracle), forward (+ backward) on the same workload."""
+    import torch
+
+    from oracle import attention as oracle
+    from trident_amd import workloads
+
+    q, k, v, d_o, mask = workloads.make_inputs(w)
+    if mask is not None:
+        mask = mask.to(w.dtype)
+    times = []
+    for rep in range(reps + 1):
+        tq, tk, tv = [x.clone().requires_grad_(w.backward) for x in (q, k, v)]
+        t0 = time.perf_counter()
+        out = oracle.sdpa_cpu(tq, tk, tv, mask, w.dropout_p, w.is_causal)
+        if w.backward:
+            out.backward(d_o)
+        dt = time.perf_counter() - t0
+        if rep > 0:
+            times.append(dt)
+    times.sort()
+    med = times[len(times) // 2]
+    return {
+        "value": round(w.flops(w.backward) / med / 1e12, 4),
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"torch CPU scaled_dot_product_attention, full {w.name} workload "
+                  f"({'fwd+bwd' if w.backward else 'fwd'}), 1 warm-up + {reps} timed reps, median {med:.3f} s; "
+                  f"os.cpu_count()={os.cpu_count()}",
+    }
+
+
+def describe(w):
+    extra = "causal" if w.is_causal else ("additive fp32 mask [B,1,S,S]" if w.masked else "plain")
+    if w.dropout_p:
+        extra += f" dropout {w.dropout_p}"
+    return f"{w.name}: {_dtype_name(w.dtype)} {extra} B={w.B} H={w.H} S={w.S} D={w.D} {'fwd+bwd' if w.backward else 'fwd'}"
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="C3")
+    ap.add_argument("--report", action="store_true", help="also print all five configurations on stderr")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build runs on one GPU; the attention path has no exchange step to "
+                 "measure across GPUs (heads shard independently). Run with --gpus 1.")
+
+    import torch
+
+    from trident_amd import workloads
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = torch.device("cuda:0")
+    w = workloads.WORKLOADS[a.workload]
+    path = Path(w, dev)
+    wall_ms, per_kernel = run_steps(path, a.steps, a.warmup)
+    dname = _dtype_name(w.dtype)
+    peak = PEAK_TFLOPS[dname]
+    flops_step = w.flops(w.backward)
+    value = flops_step / wall_ms / 1e9
+    fwd_tf = w.flops() / per_kernel["fwd"] / 1e9
+
+    dominant = max(per_kernel, key=per_kernel.get)
+    dom_flops = path.algorithmic_flops(dominant)
+    achieved = dom_flops / per_kernel[dominant] / 1e9
+    roofline = {
+        "kernel": dominant,
+        "bound": "mfma",
+        "achieved": round(achieved, 1),
+        "peak": peak,
+        "unit": "TFLOP/s",
+        "frac": round(achieved / peak, 4),
+        "traffic": MEASURED_TRAFFIC.get((w.name, dominant)),
+        "avg_launch_ms": round(per_kernel[dominant], 5),
+    }
+    result = {
+        "metric": "attention fwd & fwd+bwd TFLOP/s + % MFMA peak, bf16 causal S=4096 D=128",
+        "value": round(value, 1),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": round(wall_ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dname,
+        "data": "synthetic",
+        "config": {"workload": describe(w)},
+        "fwd_tflops": round(fwd_tf, 1),
+        "fwd_frac_of_peak": round(fwd_tf / peak, 4),
+        "fwdbwd_tflops": round(value, 1),
+        "fwdbwd_frac_of_peak": round(value / peak, 4),
+        "kernel_ms": {k: round(v, 5) for k, v in per_kernel.items()},
+        "roofline": roofline,
+    }
+    if "bwd_delta" in per_kernel:
+        nbytes = path.algorithmic_bytes("bwd_delta")
+        gbs = nbytes / per_kernel["bwd_delta"] / 1e6
+        result["delta_prepass"] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                   "frac": round(gbs / HBM_PEAK_GBS, 4)}
+    if not a.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(w)
+    print(json.dumps(result), flush=True)
+
+    if a.report:
+        for name, wl in workloads.WORKLOADS.items():
+            pth = Path(wl, dev)
+            steps = 3 if name == "C5" else 10
+            ms, pk = run_steps(pth, steps, 2)
+            pkk = PEAK_TFLOPS[_dtype_name(wl.dtype)]
+            f = wl.flops() / pk["fwd"] / 1e9
+            line = f"{describe(wl)} | fwd {pk['fwd']:.4f} ms {f:.1f} TFLOP/s ({100 * f / pkk:.1f}% of {pkk})"
+            if wl.backward:
+                t = wl.flops(True) / ms / 1e9
+                line += f" | fwd+bwd {ms:.4f} ms {t:.1f} TFLOP/s ({100 * t / pkk:.1f}%)"
+                line += " | " + " ".join(f"{k}={v:.4f}ms" for k, v in pk.items())
+            if not a.no_cpu and name != "C5":
+                cb = cpu_baseline(wl, reps=1 if name in ("C3", "C4") else 3)
+                line += f" | CPU {cb['value']} TFLOP/s on {cb['cores']} threads"
+            print(line, file=sys.stderr, flush=True)
+            del pth
+
+
+if __name__ == "__main__":
+    main()

@@ -136,6 +136,35 @@ def attention_backward(q, k, v, d_out, mask=None, dropout_p=0.0, is_causal=False
     return dq, dk, dv, dmask, delta
 
 
+def operand_abs_sums(q, k, v, d_out, mask=None, dropout_p=0.0, is_causal=False, scale=None, seed=0, offset=0, o=None):
+    """Sum of |terms| of the contractions whose left operand a 16-bit matrix-core kernel must round
+    (P for O and dV, dS for dQ and dK): A_O = |PZ| |V|, A_dV = |PZ|^T |dO|, A_dQ = scale |dS| |K|,
+    A_dK = scale |dS|^T |Q|.  Rounding P or dS to a type with unit roundoff u perturbs each output by
+    at most u * A, whatever the kernel; the parity tests add that bound to the stated atol."""
+    q, k, v, d_out = [np.asarray(x, dtype=np.float64) for x in (q, k, v, d_out)]
+    B, H, S, D = q.shape
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    a_o, a_dq, a_dk, a_dv = [np.empty_like(q) for _ in range(4)]
+    for b in range(B):
+        for h in range(H):
+            s = _scores(q[b, h], k[b, h], _mask_slice(mask, b, h), is_causal, scale)
+            p, _ = _softmax_rows(s)
+            z = _keep_scale(seed, offset, b * H + h, S, dropout_p)
+            pz = p if z is None else p * z
+            o_bh = pz @ v[b, h] if o is None else np.asarray(o[b, h], dtype=np.float64)
+            dlt = np.sum(d_out[b, h] * o_bh, axis=-1)
+            dp = d_out[b, h] @ v[b, h].T
+            if z is not None:
+                dp = dp * z
+            ds = np.abs(p * (dp - dlt[:, None]))
+            a_o[b, h] = pz @ np.abs(v[b, h])
+            a_dv[b, h] = pz.T @ np.abs(d_out[b, h])
+            a_dq[b, h] = scale * (ds @ np.abs(k[b, h]))
+            a_dk[b, h] = scale * (ds.T @ np.abs(q[b, h]))
+    return a_o, a_dq, a_dk, a_dv
+
+
 def attention_bruteforce(q, k, v, mask=None, is_causal=False, scale=None, keep_scale=None):
     """Scalar-loop forward for tiny inputs (pins the vectorised path). keep_scale: optional
     [B,H,S,S] array of Z = keep/(1-p). Returns (O, lse_natural)."""

@@ -51,9 +51,10 @@ def _check(device, dtype, q, k, v, d_o, mask=None, dropout_p=0.0, is_causal=Fals
     parity.close(o, o_ref, dtype, tag + " O")
     if d_o is not None:
         dq_r, dk_r, dv_r, dm_r, _ = parity.oracle_backward(q, k, v, d_o, want_dmask=mask_grad, o=o, **kw)
-        parity.close(dq, dq_r, dtype, tag + " dQ")
-        parity.close(dk, dk_r, dtype, tag + " dK")
-        parity.close(dv, dv_r, dtype, tag + " dV")
+        _, a_dq, a_dk, a_dv = parity.oracle_abs_sums(q, k, v, d_o, o=o, **kw)
+        parity.close(dq, dq_r, dtype, tag + " dQ", a_dq)
+        parity.close(dk, dk_r, dtype, tag + " dK", a_dk)
+        parity.close(dv, dv_r, dtype, tag + " dV", a_dv)
         if mask_grad:
             # dS is computed from the stored (rounded) O and 16-bit operands: its error budget is
             # that of the q/k/v dtype even when the mask itself is fp32
@@ -244,9 +245,10 @@ def test_config3_full_size_properties(device):
         o_ref, _ = parity.oracle_forward(q[sl], k[sl], v[sl], is_causal=True)
         dq_r, dk_r, dv_r, _, _ = parity.oracle_backward(q[sl], k[sl], v[sl], d_o[sl], is_causal=True, o=out[sl])
         parity.close(out[sl], o_ref, w.dtype, f"C3 head {b},{h} O")
-        parity.close(tq.grad[sl], dq_r, w.dtype, "C3 dQ")
-        parity.close(tk.grad[sl], dk_r, w.dtype, "C3 dK")
-        parity.close(tv.grad[sl], dv_r, w.dtype, "C3 dV")
+        _, a_dq, a_dk, a_dv = parity.oracle_abs_sums(q[sl], k[sl], v[sl], d_o[sl], is_causal=True, o=out[sl])
+        parity.close(tq.grad[sl], dq_r, w.dtype, "C3 dQ", a_dq)
+        parity.close(tk.grad[sl], dk_r, w.dtype, "C3 dK", a_dk)
+        parity.close(tv.grad[sl], dv_r, w.dtype, "C3 dV", a_dv)
     # V == 1 gives O == 1 at full size (softmax rows sum to one)
     ones = torch.ones_like(tv)
     o1 = trident.function.scaled_dot_product_attention(tq.detach(), tk.detach(), ones, is_causal=True)

@@ -300,3 +300,25 @@ def test_golden_fixture():
             np.testing.assert_allclose(val, data[f"{name}.{key}"], rtol=0, atol=1e-13)
         if dm is not None:
             np.testing.assert_allclose(dm, data[f"{name}.dmask"], rtol=0, atol=1e-13)
+
+
+def test_backward_with_saved_output_and_abs_sums():
+    """delta is defined on the output tensor handed to the backward; abs sums bound the gradients."""
+    shape = (1, 2, 12, 4)
+    q, k, v, d_o = [_rand(shape, s) for s in (1, 2, 3, 4)]
+    o, _ = oracle.attention_forward(q, k, v, is_causal=True)
+    base = oracle.attention_backward(q, k, v, d_o, is_causal=True)
+    same = oracle.attention_backward(q, k, v, d_o, is_causal=True, o=o)
+    for a, b in zip(base[:3], same[:3]):
+        np.testing.assert_allclose(a, b, atol=1e-13)
+    o2 = o + 0.5
+    dq2, dk2, dv2, _, delta2 = oracle.attention_backward(q, k, v, d_o, is_causal=True, o=o2)
+    np.testing.assert_allclose(delta2, (d_o * o2).sum(-1), atol=1e-13)
+    np.testing.assert_allclose(dv2, base[2], atol=1e-13)  # dV does not depend on delta
+    assert np.abs(dq2 - base[0]).max() > 1e-3
+    a_o, a_dq, a_dk, a_dv = oracle.operand_abs_sums(q, k, v, d_o, is_causal=True)
+    assert (np.abs(o) <= a_o + 1e-12).all() and (np.abs(base[0]) <= a_dq + 1e-12).all()
+    assert (np.abs(base[1]) <= a_dk + 1e-12).all() and (np.abs(base[2]) <= a_dv + 1e-12).all()
+    # non-negative inputs make the bound tight for O
+    o_pos, _ = oracle.attention_forward(q, k, np.abs(v), is_causal=True)
+    np.testing.assert_allclose(o_pos, a_o, atol=1e-13)

@@ -1,0 +1,353 @@
+// Backward attention on the matrix cores for fp16/bf16, D in {64,128}, S a multiple of 128
+// (replaces trident/kernel/attention.py:169-339, split in two passes so that no gradient
+// tile is ever accumulated in global memory):
+//
+//   dQ pass    one workgroup per 128 query rows (a wave owns 32), streaming key tiles of 64:
+//              S^T = K Q^T, dP^T = V dO^T, dS^T = P^T * (dP^T - delta), dQ^T += K^T dS^T
+//   dK/dV pass one workgroup per 128 keys (a wave owns 32), streaming query tiles of 64:
+//              S = Q K^T, dP = dO V^T, dV^T += dO^T P, dK^T += Q^T dS
+//
+// In both, the lane index is the row that owns the accumulators (query row resp. key), the
+// stationary operands (Q,dO resp. K,V) stay in registers as MFMA B operands, and P / dS go
+// from the accumulators of one MFMA to the B operand of the next without leaving registers.
+#include "launch.hpp"
+#include "mfma_common.hpp"
+
+namespace tri {
+namespace {
+
+constexpr int kBM = 128;  // stationary rows per workgroup
+constexpr int kBN = 64;   // streamed rows per tile
+
+enum MaskKind { kNoMask = 0, kMaskF32 = 1, kMaskT = 2 };
+
+template <typename T, int MASK>
+__device__ __forceinline__ float mask_at(const void* mask, int64_t off) {
+    if constexpr (MASK == kMaskF32) return static_cast<const float*>(mask)[off];
+    else return static_cast<float>(static_cast<const T*>(mask)[off]);
+}
+
+// ------------------------------------------------------------------------------------ dQ
+template <typename T, int D, bool CAUSAL, int MASK, bool DROPOUT>
+__global__ __launch_bounds__(256, 2) void mfma_dq_kernel(const KParams p) {
+    constexpr int kRowBytes = RowTile<D>::bytes(kBN);
+    constexpr int kTransBytes = TransTile::bytes(D);
+    constexpr int KK = D / 16;
+    constexpr int DB = D / 32;
+    __shared__ __attribute__((aligned(16))) char smem[2 * kRowBytes + kTransBytes];
+    char* sK = smem;
+    char* sV = smem + kRowBytes;
+    char* sKt = smem + 2 * kRowBytes;
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+    int bh, qt;
+    map_block(blockIdx.x, p.B * p.H, p.S / kBM, CAUSAL, &bh, &qt);
+    const int b = bh / p.H, hd = bh % p.H;
+    const int q0 = qt * kBM;
+    const int wrow0 = q0 + 32 * wave;
+    const int qrow = wrow0 + l32;
+
+    const char* qrowp = static_cast<const char*>(p.q) + (b * p.qs[0] + hd * p.qs[1] + static_cast<int64_t>(qrow) * p.qs[2]) * 2;
+    const char* gorowp = static_cast<const char*>(p.d_o) + (b * p.dos[0] + hd * p.dos[1] + static_cast<int64_t>(qrow) * p.dos[2]) * 2;
+    const char* kbase = static_cast<const char*>(p.k) + (b * p.ks[0] + hd * p.ks[1]) * 2;
+    const char* vbase = static_cast<const char*>(p.v) + (b * p.vs[0] + hd * p.vs[1]) * 2;
+    const int64_t krow_bytes = p.ks[2] * 2, vrow_bytes = p.vs[2] * 2;
+
+    u32x4 qf[KK], gf[KK];
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+        qf[kk] = *reinterpret_cast<const u32x4*>(qrowp + (2 * kk + h) * 16);
+        gf[kk] = *reinterpret_cast<const u32x4*>(gorowp + (2 * kk + h) * 16);
+    }
+    float lse = p.lse[static_cast<int64_t>(bh) * p.S + qrow];
+    if (lse == -INFINITY) lse = INFINITY;  // fully masked row: every probability is 0
+    const float dlt = p.delta[static_cast<int64_t>(bh) * p.S + qrow];
+    const float c = p.scale_log2;
+
+    f32x16 acc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) acc[db] = zero16();
+
+    const int n_tiles = CAUSAL ? (q0 + kBM) / kBN : p.S / kBN;
+    TransStage<T, D> kst;
+    RowStage<D> vst;
+    kst.load(kbase, krow_bytes, tid);
+    vst.load(vbase, vrow_bytes, tid);
+
+    for (int j = 0; j < n_tiles; ++j) {
+        const int t0 = j * kBN;
+        kst.store_rows(sK, tid);
+        kst.store(sKt, tid);
+        vst.store(sV, tid);
+        __syncthreads();
+        if (j + 1 < n_tiles) {
+            kst.load(kbase + (t0 + kBN) * krow_bytes, krow_bytes, tid);
+            vst.load(vbase + (t0 + kBN) * vrow_bytes, vrow_bytes, tid);
+        }
+        const bool active = !CAUSAL || t0 <= wrow0 + 31;
+        if (active) {
+            const bool diag = CAUSAL && t0 + kBN - 1 > wrow0;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                float mk[MASK != kNoMask ? 16 : 1];
+                if constexpr (MASK != kNoMask) {
+                    const int64_t mrow = b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(qrow) * p.ms[2] + t0 + 32 * kb;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) mk[i] = mask_at<T, MASK>(p.mask, mrow + c_row(i, h));
+                }
+                f32x16 st = zero16(), dpt = zero16();
+#pragma unroll
+                for (int kk = 0; kk < KK; ++kk) {
+                    const u32x4 a = lds_read16(sK, RowTile<D>::off(32 * kb + l32, 2 * kk + h));
+                    st = Mma<T>::run(a, qf[kk], st);
+                }
+#pragma unroll
+                for (int kk = 0; kk < KK; ++kk) {
+                    const u32x4 a = lds_read16(sV, RowTile<D>::off(32 * kb + l32, 2 * kk + h));
+                    dpt = Mma<T>::run(a, gf[kk], dpt);
+                }
+                float ds[16];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int key = t0 + 32 * kb + c_row(i, h);
+                    float x = st[i] * c;
+                    if constexpr (MASK != kNoMask) x = fmaf(mk[i], kLog2e, x);
+                    float pr = fast_exp2(x - lse);
+                    if (diag) pr = key <= qrow ? pr : 0.f;
+                    ds[i] = pr;
+                }
+                if constexpr (DROPOUT) {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const uint32_t w = dropout_word(p, bh, qrow, t0 + 32 * kb + 8 * g + 4 * h);
+#pragma unroll
+                        for (int bb = 0; bb < 4; ++bb) {
+                            const bool keep = static_cast<int>((w >> (8 * bb)) & 0xffu) >= p.thr8;
+                            dpt[4 * g + bb] = keep ? dpt[4 * g + bb] * p.zscale : 0.f;
+                        }
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) ds[i] *= dpt[i] - dlt;
+#pragma unroll
+                for (int g = 0; g < 2; ++g) {
+                    const u32x4 bop = pack8<T>(&ds[8 * g]);
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) {
+                        const u32x4 a = lds_read16(sKt, TransTile::read_off(32 * db + l32, 2 * kb + g, h));
+                        acc[db] = Mma<T>::run(a, bop, acc[db]);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    char* out = static_cast<char*>(p.dq) + (b * p.dqs[0] + hd * p.dqs[1] + static_cast<int64_t>(qrow) * p.dqs[2]) * 2;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            u32x2 v;
+            v.x = Mma<T>::pack2(acc[db][4 * g + 0] * p.scale, acc[db][4 * g + 1] * p.scale);
+            v.y = Mma<T>::pack2(acc[db][4 * g + 2] * p.scale, acc[db][4 * g + 3] * p.scale);
+            *reinterpret_cast<u32x2*>(out + (32 * db + 8 * g + 4 * h) * 2) = v;
+        }
+}
+
+// --------------------------------------------------------------------------------- dK, dV
+template <typename T, int D, bool CAUSAL, int MASK, bool DROPOUT>
+__global__ __launch_bounds__(256, 2) void mfma_dkdv_kernel(const KParams p) {
+    constexpr int kRowBytes = RowTile<D>::bytes(kBN);
+    constexpr int kTransBytes = TransTile::bytes(D);
+    constexpr int KK = D / 16;
+    constexpr int DB = D / 32;
+    __shared__ __attribute__((aligned(16))) char smem[2 * kRowBytes + 2 * kTransBytes + 2 * kBN * 4];
+    char* sQ = smem;
+    char* sG = smem + kRowBytes;
+    char* sQt = smem + 2 * kRowBytes;
+    char* sGt = sQt + kTransBytes;
+    float* sLse = reinterpret_cast<float*>(sGt + kTransBytes);
+    float* sDelta = sLse + kBN;
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+    int bh, kt;
+    map_block(blockIdx.x, p.B * p.H, p.S / kBM, false, &bh, &kt);
+    const int b = bh / p.H, hd = bh % p.H;
+    const int k0 = kt * kBM;
+    const int wkey0 = k0 + 32 * wave;
+    const int key = wkey0 + l32;
+
+    const char* krowp = static_cast<const char*>(p.k) + (b * p.ks[0] + hd * p.ks[1] + static_cast<int64_t>(key) * p.ks[2]) * 2;
+    const char* vrowp = static_cast<const char*>(p.v) + (b * p.vs[0] + hd * p.vs[1] + static_cast<int64_t>(key) * p.vs[2]) * 2;
+    const char* qbase = static_cast<const char*>(p.q) + (b * p.qs[0] + hd * p.qs[1]) * 2;
+    const char* gbase = static_cast<const char*>(p.d_o) + (b * p.dos[0] + hd * p.dos[1]) * 2;
+    const int64_t qrow_bytes = p.qs[2] * 2, grow_bytes = p.dos[2] * 2;
+    const float* lse_base = p.lse + static_cast<int64_t>(bh) * p.S;
+    const float* delta_base = p.delta + static_cast<int64_t>(bh) * p.S;
+
+    u32x4 kf[KK], vf[KK];
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+        kf[kk] = *reinterpret_cast<const u32x4*>(krowp + (2 * kk + h) * 16);
+        vf[kk] = *reinterpret_cast<const u32x4*>(vrowp + (2 * kk + h) * 16);
+    }
+    const float c = p.scale_log2;
+
+    f32x16 dk[DB], dv[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+        dk[db] = zero16();
+        dv[db] = zero16();
+    }
+
+    const int j_begin = CAUSAL ? k0 / kBN : 0;
+    const int n_tiles = p.S / kBN;
+    for (int j = j_begin; j < n_tiles; ++j) {
+        const int r0 = j * kBN;
+        {
+            TransStage<T, D> st;
+            st.load(qbase + r0 * qrow_bytes, qrow_bytes, tid);
+            st.store_rows(sQ, tid);
+            st.store(sQt, tid);
+            st.load(gbase + r0 * grow_bytes, grow_bytes, tid);
+            st.store_rows(sG, tid);
+            st.store(sGt, tid);
+            if (tid < kBN) {
+                float l = lse_base[r0 + tid];
+                sLse[tid] = l == -INFINITY ? INFINITY : l;
+                sDelta[tid] = delta_base[r0 + tid];
+            }
+        }
+        __syncthreads();
+        const bool active = !CAUSAL || r0 + kBN - 1 >= wkey0;
+        if (active) {
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb) {
+                const int rb = r0 + 32 * qb;  // first query row of this block
+                if (CAUSAL && rb + 31 < wkey0) continue;
+                const bool diag = CAUSAL && rb < wkey0 + 31;
+                float mk[MASK != kNoMask ? 16 : 1];
+                if constexpr (MASK != kNoMask) {
+                    const int64_t mbase = b * p.ms[0] + hd * p.ms[1] + key;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i)
+                        mk[i] = mask_at<T, MASK>(p.mask, mbase + static_cast<int64_t>(rb + c_row(i, h)) * p.ms[2]);
+                }
+                f32x16 s = zero16(), dp = zero16();
+#pragma unroll
+                for (int kk = 0; kk < KK; ++kk) {
+                    const u32x4 a = lds_read16(sQ, RowTile<D>::off(32 * qb + l32, 2 * kk + h));
+                    s = Mma<T>::run(a, kf[kk], s);
+                }
+#pragma unroll
+                for (int kk = 0; kk < KK; ++kk) {
+                    const u32x4 a = lds_read16(sG, RowTile<D>::off(32 * qb + l32, 2 * kk + h));
+                    dp = Mma<T>::run(a, vf[kk], dp);
+                }
+                float pr[16], ds[16];
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + 32 * qb + 8 * g + 4 * h);
+                    const f32x4 d4 = *reinterpret_cast<const f32x4*>(sDelta + 32 * qb + 8 * g + 4 * h);
+                    uint32_t dw[4];
+                    if constexpr (DROPOUT) {
+                        const Philox4 r = dropout_block(p, bh, (rb + 8 * g + 4 * h) >> 2, key >> 2);
+#pragma unroll
+                        for (int bb = 0; bb < 4; ++bb) dw[bb] = (r.w[bb] >> (8 * (key & 3))) & 0xffu;
+                    }
+#pragma unroll
+                    for (int bb = 0; bb < 4; ++bb) {
+                        const int i = 4 * g + bb;
+                        const int qrow = rb + c_row(i, h);
+                        float x = s[i] * c;
+                        if constexpr (MASK != kNoMask) x = fmaf(mk[i], kLog2e, x);
+                        float pv = fast_exp2(x - l4[bb]);
+                        if (diag) pv = key <= qrow ? pv : 0.f;
+                        float dpv = dp[i];
+                        if constexpr (DROPOUT) {
+                            const bool keep = static_cast<int>(dw[bb]) >= p.thr8;
+                            dpv = keep ? dpv * p.zscale : 0.f;
+                            pr[i] = keep ? pv * p.zscale : 0.f;
+                        } else {
+                            pr[i] = pv;
+                        }
+                        ds[i] = pv * (dpv - d4[bb]);
+                    }
+                }
+#pragma unroll
+                for (int g = 0; g < 2; ++g) {
+                    const u32x4 pb = pack8<T>(&pr[8 * g]);
+                    const u32x4 sb = pack8<T>(&ds[8 * g]);
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) {
+                        const u32x4 a = lds_read16(sGt, TransTile::read_off(32 * db + l32, 2 * qb + g, h));
+                        dv[db] = Mma<T>::run(a, pb, dv[db]);
+                    }
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) {
+                        const u32x4 a = lds_read16(sQt, TransTile::read_off(32 * db + l32, 2 * qb + g, h));
+                        dk[db] = Mma<T>::run(a, sb, dk[db]);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    char* dkrow = static_cast<char*>(p.dk) + (b * p.dks[0] + hd * p.dks[1] + static_cast<int64_t>(key) * p.dks[2]) * 2;
+    char* dvrow = static_cast<char*>(p.dv) + (b * p.dvs[0] + hd * p.dvs[1] + static_cast<int64_t>(key) * p.dvs[2]) * 2;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            u32x2 a, e;
+            a.x = Mma<T>::pack2(dk[db][4 * g + 0] * p.scale, dk[db][4 * g + 1] * p.scale);
+            a.y = Mma<T>::pack2(dk[db][4 * g + 2] * p.scale, dk[db][4 * g + 3] * p.scale);
+            e.x = Mma<T>::pack2(dv[db][4 * g + 0], dv[db][4 * g + 1]);
+            e.y = Mma<T>::pack2(dv[db][4 * g + 2], dv[db][4 * g + 3]);
+            *reinterpret_cast<u32x2*>(dkrow + (32 * db + 8 * g + 4 * h) * 2) = a;
+            *reinterpret_cast<u32x2*>(dvrow + (32 * db + 8 * g + 4 * h) * 2) = e;
+        }
+}
+
+// ---------------------------------------------------------------------------------- launch
+template <int WHICH, typename T, int D, bool CAUSAL, int MASK>
+int launch_bwd_dropout(const KParams& p, hipStream_t stream) {
+    const dim3 grid(p.B * p.H * (p.S / kBM)), block(256);
+    if (WHICH == kMfmaDq) {
+        if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dq_kernel<T, D, CAUSAL, MASK, true>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((mfma_dq_kernel<T, D, CAUSAL, MASK, false>), grid, block, 0, stream, p);
+    } else {
+        if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, CAUSAL, MASK, true>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, CAUSAL, MASK, false>), grid, block, 0, stream, p);
+    }
+    return static_cast<int>(hipGetLastError());
+}
+
+template <int WHICH, typename T, int D>
+int launch_bwd_variant(int dtype, const KParams& p, hipStream_t stream) {
+    if (p.causal) return launch_bwd_dropout<WHICH, T, D, true, kNoMask>(p, stream);
+    if (p.mask == nullptr) return launch_bwd_dropout<WHICH, T, D, false, kNoMask>(p, stream);
+    if (p.mask_dtype == TRI_ATTN_F32) return launch_bwd_dropout<WHICH, T, D, false, kMaskF32>(p, stream);
+    if (p.mask_dtype == dtype) return launch_bwd_dropout<WHICH, T, D, false, kMaskT>(p, stream);
+    return TRI_ATTN_EDTYPE;
+}
+
+template <int WHICH>
+int launch_bwd(int dtype, const KParams& p, hipStream_t stream) {
+    if (dtype == TRI_ATTN_BF16)
+        return p.D == 128 ? launch_bwd_variant<WHICH, bf16_t, 128>(dtype, p, stream)
+                          : launch_bwd_variant<WHICH, bf16_t, 64>(dtype, p, stream);
+    return p.D == 128 ? launch_bwd_variant<WHICH, f16_t, 128>(dtype, p, stream)
+                      : launch_bwd_variant<WHICH, f16_t, 64>(dtype, p, stream);
+}
+
+}  // namespace
+
+int launch_mfma_dq(int dtype, const KParams& p, hipStream_t stream) { return launch_bwd<kMfmaDq>(dtype, p, stream); }
+int launch_mfma_dkdv(int dtype, const KParams& p, hipStream_t stream) { return launch_bwd<kMfmaDkdv>(dtype, p, stream); }
+
+}  // namespace tri

@@ -165,6 +165,23 @@ struct TransStage {
             }
         }
     }
+    // the same registers written row-major into a RowTile<D>
+    __device__ __forceinline__ void store_rows(char* smem, int tid) const {
+        const int rq = tid >> 4, c = tid & 15;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            const int off = (4 * rq + a) * RowTile<D>::kStride + c * kCols * 2;
+            if constexpr (kWords == 4) {
+                u32x4 v;
+                v.x = r[a][0]; v.y = r[a][1]; v.z = r[a][2]; v.w = r[a][3];
+                lds_write16(smem, off, v);
+            } else {
+                u32x2 v;
+                v.x = r[a][0]; v.y = r[a][1];
+                lds_write8(smem, off, v);
+            }
+        }
+    }
     __device__ __forceinline__ void store(char* smem, int tid) const {
         const int rq = tid >> 4, c = tid & 15;
 #pragma unroll

@@ -63,15 +63,15 @@ bool mfma_supported(int which, int dtype, const KParams& p) {
         case kMfmaFwd:
             return aligned16(p.o) && strides8(p.os);
         case kMfmaDkdv:
+            return aligned16(p.d_o) && strides8(p.dos) && aligned16(p.dk) && strides8(p.dks) && aligned16(p.dv) &&
+                   strides8(p.dvs);
         case kMfmaDq:
-            return false;
+            // the mask gradient is written by the generic dQ kernel
+            return p.dmask == nullptr && aligned16(p.d_o) && strides8(p.dos) && aligned16(p.dq) && strides8(p.dqs);
         default:
             return false;
     }
 }
-
-int launch_mfma_dq(int, const KParams&, hipStream_t) { return TRI_ATTN_ESHAPE; }
-int launch_mfma_dkdv(int, const KParams&, hipStream_t) { return TRI_ATTN_ESHAPE; }
 
 int launch_delta(int dtype, const KParams& p, hipStream_t stream) {
     const bool vec = (dtype == TRI_ATTN_F16 || dtype == TRI_ATTN_BF16) && (p.D == 64 || p.D == 128) &&
