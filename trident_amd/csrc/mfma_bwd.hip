@@ -74,6 +74,8 @@ __global__ __launch_bounds__(256, 2) void mfma_dq_kernel(const KParams p) {
     RowStage<D> vst;
     kst.load(kbase, krow_bytes, tid);
     vst.load(vbase, vrow_bytes, tid);
+    // all loads issued so far have landed; otherwise the compiler waits on vmcnt in the loop
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
 
     for (int j = 0; j < n_tiles; ++j) {
         const int t0 = j * kBN;
@@ -205,6 +207,7 @@ __global__ __launch_bounds__(256, 2) void mfma_dkdv_kernel(const KParams p) {
 
     const int j_begin = CAUSAL ? k0 / kBN : 0;
     const int n_tiles = p.S / kBN;
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): K/V fragments are in registers
     for (int j = j_begin; j < n_tiles; ++j) {
         const int r0 = j * kBN;
         {

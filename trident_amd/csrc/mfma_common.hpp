@@ -40,6 +40,11 @@ struct Mma<bf16_t> {
     }
     static __device__ __forceinline__ float lo(uint32_t w) { return __uint_as_float(w << 16); }
     static __device__ __forceinline__ float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+    // acc + lo(w) + hi(w) in one instruction (v_dot2c_f32_bf16 against (1, 1))
+    static __device__ __forceinline__ float add_pair(uint32_t w, float acc) {
+        const bf16x2 ones = {static_cast<bf16_t>(1.0f), static_cast<bf16_t>(1.0f)};
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w), ones, acc, false);
+    }
 };
 template <>
 struct Mma<f16_t> {
@@ -56,6 +61,10 @@ struct Mma<f16_t> {
     }
     static __device__ __forceinline__ float hi(uint32_t w) {
         return static_cast<float>(__builtin_bit_cast(f16x2, w)[1]);
+    }
+    static __device__ __forceinline__ float add_pair(uint32_t w, float acc) {
+        const f16x2 ones = {static_cast<f16_t>(1.0f), static_cast<f16_t>(1.0f)};
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, w), ones, acc, false);
     }
 };
 
@@ -144,15 +153,22 @@ struct RowStage {
 };
 
 // Global -> registers -> LDS staging of one [64][D] tile into a TransTile: thread (rq, c) holds
-// source rows 4rq..4rq+3, columns c*D/16 .. (c+1)*D/16-1 (16 lanes cover one source row, so
-// the global loads stay row-contiguous).
+// source rows 4rq..4rq+3, columns c*D/16 .. (c+1)*D/16-1. Eight consecutive lanes cover half a
+// source row (one 128- or 64-byte segment of the global load); the 16 lanes that an 8-byte LDS
+// write handles per clock are 8 column chunks x 2 row quads whose slots differ in the 8-byte
+// half, so with the XOR swizzle they fall into 16 different bank pairs.
 template <typename T, int D>
 struct TransStage {
     static constexpr int kCols = D / 16;      // 8 for D=128 (16-byte loads), 4 for D=64 (8-byte loads)
     static constexpr int kWords = kCols / 2;
     uint32_t r[4][kWords];
+    static __device__ __forceinline__ int col_chunk(int tid) { return (tid & 7) | (((tid >> 4) & 1) << 3); }
+    static __device__ __forceinline__ int row_quad(int tid) {
+        const int rest = tid >> 5;
+        return ((rest >> 1) << 2) | (((tid >> 3) & 1) << 1) | (rest & 1);
+    }
     __device__ __forceinline__ void load(const char* base, int64_t row_stride_bytes, int tid) {
-        const int rq = tid >> 4, c = tid & 15;
+        const int rq = row_quad(tid), c = col_chunk(tid);
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
             const char* src = base + (4 * rq + a) * row_stride_bytes + c * kCols * 2;
@@ -167,7 +183,7 @@ struct TransStage {
     }
     // the same registers written row-major into a RowTile<D>
     __device__ __forceinline__ void store_rows(char* smem, int tid) const {
-        const int rq = tid >> 4, c = tid & 15;
+        const int rq = row_quad(tid), c = col_chunk(tid);
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
             const int off = (4 * rq + a) * RowTile<D>::kStride + c * kCols * 2;
@@ -183,7 +199,7 @@ struct TransStage {
         }
     }
     __device__ __forceinline__ void store(char* smem, int tid) const {
-        const int rq = tid >> 4, c = tid & 15;
+        const int rq = row_quad(tid), c = col_chunk(tid);
 #pragma unroll
         for (int wd = 0; wd < kWords; ++wd) {
             // even column: low halves of the four rows; odd column: high halves

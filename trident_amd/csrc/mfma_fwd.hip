@@ -15,6 +15,7 @@ namespace {
 
 constexpr int kBM = 128;  // query rows per workgroup
 constexpr int kBN = 64;   // keys per tile
+constexpr float kTau = 8.f;  // lazy-rescale threshold, log2 domain
 
 enum MaskKind { kNoMask = 0, kMaskF32 = 1, kMaskT = 2 };
 
@@ -60,6 +61,9 @@ __global__ __launch_bounds__(256, 2) void mfma_fwd_kernel(const KParams p) {
     vst.load(vbase, vrow_bytes, tid);
     kst.store(smem, tid);
     vst.store(smem + kKBytes, tid);
+    // every global load issued so far (Q fragments, first tile) has landed: without this the
+    // compiler keeps waiting on vmcnt inside the loop and serialises each tile's prefetch
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
 
     for (int j = 0; j < n_tiles; ++j) {
@@ -91,18 +95,38 @@ __global__ __launch_bounds__(256, 2) void mfma_fwd_kernel(const KParams p) {
                     }
                 }
             }
-            // S^T = K Q^T
+            // S^T = K Q^T with the A fragments requested kAhead MFMAs before their use, so that
+            // the LDS latency overlaps the matrix pipe instead of stalling every MFMA pair
+            {
+                constexpr int kSteps = 2 * KK, kAhead = 8;
+                u32x4 ring[kAhead];
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                f32x16 st = zero16();
+                for (int s = 0; s < kAhead; ++s)
+                    ring[s] = lds_read16(sK, RowTile<D>::off(32 * (s / KK) + l32, 2 * (s % KK) + h));
+                __builtin_amdgcn_sched_barrier(0);
+                f32x16 st[2] = {zero16(), zero16()};
 #pragma unroll
-                for (int kk = 0; kk < KK; ++kk) {
-                    const u32x4 a = lds_read16(sK, RowTile<D>::off(32 * kb + l32, 2 * kk + h));
-                    st = Mma<T>::run(a, qf[kk], st);
+                for (int s = 0; s < kSteps; ++s) {
+                    st[s / KK] = Mma<T>::run(ring[s % kAhead], qf[s % KK], st[s / KK]);
+                    if (s + kAhead < kSteps) {
+                        const int n = s + kAhead;
+                        ring[s % kAhead] = lds_read16(sK, RowTile<D>::off(32 * (n / KK) + l32, 2 * (n % KK) + h));
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
 #pragma unroll
-                for (int i = 0; i < 16; ++i) x[16 * kb + i] = st[i];
+                for (int i = 0; i < 16; ++i) {
+                    x[i] = st[0][i];
+                    x[16 + i] = st[1][i];
+                }
             }
+            // first V^T fragments of the second product: requested now, they arrive during the softmax
+            constexpr int kPvSteps = 4 * DB, kPvAhead = 8;
+            u32x4 vring[kPvAhead];
+#pragma unroll
+            for (int s = 0; s < kPvAhead; ++s)
+                vring[s] = lds_read16(sV, TransTile::read_off(32 * (s % DB) + l32, s / DB, h));
+            __builtin_amdgcn_sched_barrier(0);
             // scores in the log2 domain; without a mask the scale is folded into the exponent
             if constexpr (MASK != kNoMask) {
 #pragma unroll
@@ -120,23 +144,30 @@ __global__ __launch_bounds__(256, 2) void mfma_fwd_kernel(const KParams p) {
             for (int e = 1; e < 32; ++e) mx = fmaxf(mx, x[e]);
             mx = fmaxf(mx, xor32(mx));
             if constexpr (MASK == kNoMask) mx *= c;
-            const float m_new = fmaxf(m, mx);
-            const float m_use = m_new == -INFINITY ? 0.f : m_new;
-            const float alpha = fast_exp2(m - m_use);
-            float psum = 0.f;
+            // Lazy rescaling: m is the reference exponent of l and of the O accumulators, not
+            // necessarily the running maximum. It is only moved (and O rescaled) when some row of
+            // the wave outgrew it by more than 2^kTau; until then probabilities may exceed 1 by
+            // that factor, which fp32 sums and 16-bit P hold without loss.
+            if (__builtin_amdgcn_ballot_w64(mx > m + kTau) != 0) {
+                const float m_new = fmaxf(m, mx);
+                const float alpha = fast_exp2(m - (m_new == -INFINITY ? 0.f : m_new));
+                l *= alpha;
+                m = m_new;
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) oacc[db][i] *= alpha;
+            }
+            const float m_use = m == -INFINITY ? 0.f : m;
 #pragma unroll
             for (int e = 0; e < 32; ++e) {
                 if constexpr (MASK == kNoMask) x[e] = fast_exp2(fmaf(x[e], c, -m_use));
                 else x[e] = fast_exp2(x[e] - m_use);
-                psum += x[e];
             }
-            l = fmaf(l, alpha, psum);
-            m = m_new;
-#pragma unroll
-            for (int db = 0; db < DB; ++db)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) oacc[db][i] *= alpha;
+            float psum = 0.f;
             if constexpr (DROPOUT) {
+#pragma unroll
+                for (int e = 0; e < 32; ++e) psum += x[e];
 #pragma unroll
                 for (int g = 0; g < 8; ++g) {
                     const int key0 = t0 + 32 * (g >> 2) + 8 * (g & 3) + 4 * h;
@@ -148,16 +179,30 @@ __global__ __launch_bounds__(256, 2) void mfma_fwd_kernel(const KParams p) {
                     }
                 }
             }
-            // O^T += V^T P^T
+            // O^T += V^T P^T; without dropout the row sum is taken from the rounded P that is
+            // actually multiplied with V, two values per instruction
+            u32x4 pb[4];
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) {
-                const u32x4 pb = pack8<T>(&x[8 * ks]);
-#pragma unroll
-                for (int db = 0; db < DB; ++db) {
-                    const u32x4 a = lds_read16(sV, TransTile::read_off(32 * db + l32, ks, h));
-                    oacc[db] = Mma<T>::run(a, pb, oacc[db]);
+                pb[ks] = pack8<T>(&x[8 * ks]);
+                if constexpr (!DROPOUT) {
+                    psum = Mma<T>::add_pair(pb[ks].x, psum);
+                    psum = Mma<T>::add_pair(pb[ks].y, psum);
+                    psum = Mma<T>::add_pair(pb[ks].z, psum);
+                    psum = Mma<T>::add_pair(pb[ks].w, psum);
                 }
             }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s = 0; s < kPvSteps; ++s) {
+                oacc[s % DB] = Mma<T>::run(vring[s % kPvAhead], pb[s / DB], oacc[s % DB]);
+                if (s + kPvAhead < kPvSteps) {
+                    const int n = s + kPvAhead;
+                    vring[s % kPvAhead] = lds_read16(sV, TransTile::read_off(32 * (n % DB) + l32, n / DB, h));
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            l += psum;
         }
         if (more) {
             char* nK = smem + ((j + 1) & 1) * kStageBytes;
