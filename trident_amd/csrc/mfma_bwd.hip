@@ -42,7 +42,7 @@ __global__ __launch_bounds__(256, 2) void mfma_dq_kernel(const KParams p) {
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
     int bh, qt;
-    map_block(blockIdx.x, p.B * p.H, p.S / kBM, CAUSAL, &bh, &qt);
+    map_block(blockIdx.x, p.B * p.H, p.S / kBM, CAUSAL ? kHeavyLast : kUniformTiles, &bh, &qt);
     const int b = bh / p.H, hd = bh % p.H;
     const int q0 = qt * kBM;
     const int wrow0 = q0 + 32 * wave;
@@ -70,22 +70,21 @@ __global__ __launch_bounds__(256, 2) void mfma_dq_kernel(const KParams p) {
     for (int db = 0; db < DB; ++db) acc[db] = zero16();
 
     const int n_tiles = CAUSAL ? (q0 + kBM) / kBN : p.S / kBN;
-    TransStage<T, D> kst;
-    RowStage<D> vst;
-    kst.load(kbase, krow_bytes, tid);
-    vst.load(vbase, vrow_bytes, tid);
+    uint32_t kst[StageRegs<D>::kCount], vst[StageRegs<D>::kCount];
+    TransStage<D>::load(kst, kbase, krow_bytes, tid);
+    RowStage<D>::load(vst, vbase, vrow_bytes, tid);
     // all loads issued so far have landed; otherwise the compiler waits on vmcnt in the loop
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
 
     for (int j = 0; j < n_tiles; ++j) {
         const int t0 = j * kBN;
-        kst.store_rows(sK, tid);
-        kst.store(sKt, tid);
-        vst.store(sV, tid);
+        TransStage<D>::store_rows(kst, sK, tid);
+        TransStage<D>::store(kst, sKt, tid);
+        RowStage<D>::store(vst, sV, tid);
         __syncthreads();
         if (j + 1 < n_tiles) {
-            kst.load(kbase + (t0 + kBN) * krow_bytes, krow_bytes, tid);
-            vst.load(vbase + (t0 + kBN) * vrow_bytes, vrow_bytes, tid);
+            TransStage<D>::load(kst, kbase + (t0 + kBN) * krow_bytes, krow_bytes, tid);
+            RowStage<D>::load(vst, vbase + (t0 + kBN) * vrow_bytes, vrow_bytes, tid);
         }
         const bool active = !CAUSAL || t0 <= wrow0 + 31;
         if (active) {
@@ -176,7 +175,7 @@ __global__ __launch_bounds__(256, 2) void mfma_dkdv_kernel(const KParams p) {
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
     int bh, kt;
-    map_block(blockIdx.x, p.B * p.H, p.S / kBM, false, &bh, &kt);
+    map_block(blockIdx.x, p.B * p.H, p.S / kBM, CAUSAL ? kHeavyFirst : kUniformTiles, &bh, &kt);
     const int b = bh / p.H, hd = bh % p.H;
     const int k0 = kt * kBM;
     const int wkey0 = k0 + 32 * wave;
@@ -211,13 +210,13 @@ __global__ __launch_bounds__(256, 2) void mfma_dkdv_kernel(const KParams p) {
     for (int j = j_begin; j < n_tiles; ++j) {
         const int r0 = j * kBN;
         {
-            TransStage<T, D> st;
-            st.load(qbase + r0 * qrow_bytes, qrow_bytes, tid);
-            st.store_rows(sQ, tid);
-            st.store(sQt, tid);
-            st.load(gbase + r0 * grow_bytes, grow_bytes, tid);
-            st.store_rows(sG, tid);
-            st.store(sGt, tid);
+            uint32_t st[StageRegs<D>::kCount];
+            TransStage<D>::load(st, qbase + r0 * qrow_bytes, qrow_bytes, tid);
+            TransStage<D>::store_rows(st, sQ, tid);
+            TransStage<D>::store(st, sQt, tid);
+            TransStage<D>::load(st, gbase + r0 * grow_bytes, grow_bytes, tid);
+            TransStage<D>::store_rows(st, sG, tid);
+            TransStage<D>::store(st, sGt, tid);
             if (tid < kBN) {
                 float l = lse_base[r0 + tid];
                 sLse[tid] = l == -INFINITY ? INFINITY : l;

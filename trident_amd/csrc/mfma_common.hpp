@@ -128,86 +128,98 @@ __device__ __forceinline__ u32x4 lds_read16(const char* smem, int off) {
 __device__ __forceinline__ void lds_write16(char* smem, int off, u32x4 v) { *reinterpret_cast<u32x4*>(smem + off) = v; }
 __device__ __forceinline__ void lds_write8(char* smem, int off, u32x2 v) { *reinterpret_cast<u32x2*>(smem + off) = v; }
 
-// Global -> registers -> LDS staging of one [64][D] tile by 256 threads, row-major target.
+// ---------------------------------------------------------------- HBM -> registers -> LDS staging
+// One [64][D] tile of 16-bit elements is moved by 256 threads, D/8 registers each. Both layouts
+// below work on the same raw register array, so a wave that stages K and a wave that stages V
+// can share one buffer in code that serves both roles.
+template <int D>
+struct StageRegs {
+    static constexpr int kCount = D / 8;  // 16 for D=128, 8 for D=64
+};
+
+// Row-major target (RowTile<D>): thread t holds 16-byte chunks t, t+256, ... of the tile.
 template <int D>
 struct RowStage {
     static constexpr int kChunksPerRow = D / 8;
     static constexpr int kPerThread = 64 * kChunksPerRow / 256;  // 4 for D=128, 2 for D=64
-    u32x4 r[kPerThread];
-    __device__ __forceinline__ void load(const char* base, int64_t row_stride_bytes, int tid) {
+    static __device__ __forceinline__ void load(uint32_t (&r)[StageRegs<D>::kCount], const char* base,
+                                                int64_t row_stride_bytes, int tid) {
 #pragma unroll
         for (int i = 0; i < kPerThread; ++i) {
             const int g = tid + 256 * i;
             const int row = g / kChunksPerRow, c = g % kChunksPerRow;
-            r[i] = *reinterpret_cast<const u32x4*>(base + row * row_stride_bytes + c * 16);
+            const u32x4 v = *reinterpret_cast<const u32x4*>(base + row * row_stride_bytes + c * 16);
+            r[4 * i + 0] = v.x; r[4 * i + 1] = v.y; r[4 * i + 2] = v.z; r[4 * i + 3] = v.w;
         }
     }
-    __device__ __forceinline__ void store(char* smem, int tid) const {
+    static __device__ __forceinline__ void store(const uint32_t (&r)[StageRegs<D>::kCount], char* smem, int tid) {
 #pragma unroll
         for (int i = 0; i < kPerThread; ++i) {
             const int g = tid + 256 * i;
             const int row = g / kChunksPerRow, c = g % kChunksPerRow;
-            lds_write16(smem, RowTile<D>::off(row, c), r[i]);
+            u32x4 v;
+            v.x = r[4 * i + 0]; v.y = r[4 * i + 1]; v.z = r[4 * i + 2]; v.w = r[4 * i + 3];
+            lds_write16(smem, RowTile<D>::off(row, c), v);
         }
     }
 };
 
-// Global -> registers -> LDS staging of one [64][D] tile into a TransTile: thread (rq, c) holds
-// source rows 4rq..4rq+3, columns c*D/16 .. (c+1)*D/16-1. Eight consecutive lanes cover half a
-// source row (one 128- or 64-byte segment of the global load); the 16 lanes that an 8-byte LDS
-// write handles per clock are 8 column chunks x 2 row quads whose slots differ in the 8-byte
-// half, so with the XOR swizzle they fall into 16 different bank pairs.
-template <typename T, int D>
+// Transposed target (TransTile): thread (rq, c) holds source rows 4rq..4rq+3, columns
+// c*D/16 .. (c+1)*D/16-1 in registers [a*kWords + w]. Eight consecutive lanes cover half a source
+// row (one 128- or 64-byte segment of the global load); the 16 lanes that an 8-byte LDS write
+// handles per clock are 8 column chunks x 2 row quads whose slots differ in the 8-byte half, so
+// with the XOR swizzle they fall into 16 different bank pairs. The same registers can also be
+// written row-major (store_rows) when a kernel needs both forms of a tile.
+template <int D>
 struct TransStage {
     static constexpr int kCols = D / 16;      // 8 for D=128 (16-byte loads), 4 for D=64 (8-byte loads)
     static constexpr int kWords = kCols / 2;
-    uint32_t r[4][kWords];
     static __device__ __forceinline__ int col_chunk(int tid) { return (tid & 7) | (((tid >> 4) & 1) << 3); }
     static __device__ __forceinline__ int row_quad(int tid) {
         const int rest = tid >> 5;
         return ((rest >> 1) << 2) | (((tid >> 3) & 1) << 1) | (rest & 1);
     }
-    __device__ __forceinline__ void load(const char* base, int64_t row_stride_bytes, int tid) {
+    static __device__ __forceinline__ void load(uint32_t (&r)[StageRegs<D>::kCount], const char* base,
+                                                int64_t row_stride_bytes, int tid) {
         const int rq = row_quad(tid), c = col_chunk(tid);
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
             const char* src = base + (4 * rq + a) * row_stride_bytes + c * kCols * 2;
             if constexpr (kWords == 4) {
                 const u32x4 v = *reinterpret_cast<const u32x4*>(src);
-                r[a][0] = v.x; r[a][1] = v.y; r[a][2] = v.z; r[a][3] = v.w;
+                r[4 * a + 0] = v.x; r[4 * a + 1] = v.y; r[4 * a + 2] = v.z; r[4 * a + 3] = v.w;
             } else {
                 const u32x2 v = *reinterpret_cast<const u32x2*>(src);
-                r[a][0] = v.x; r[a][1] = v.y;
+                r[2 * a + 0] = v.x; r[2 * a + 1] = v.y;
             }
         }
     }
-    // the same registers written row-major into a RowTile<D>
-    __device__ __forceinline__ void store_rows(char* smem, int tid) const {
+    static __device__ __forceinline__ void store_rows(const uint32_t (&r)[StageRegs<D>::kCount], char* smem, int tid) {
         const int rq = row_quad(tid), c = col_chunk(tid);
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
             const int off = (4 * rq + a) * RowTile<D>::kStride + c * kCols * 2;
             if constexpr (kWords == 4) {
                 u32x4 v;
-                v.x = r[a][0]; v.y = r[a][1]; v.z = r[a][2]; v.w = r[a][3];
+                v.x = r[4 * a + 0]; v.y = r[4 * a + 1]; v.z = r[4 * a + 2]; v.w = r[4 * a + 3];
                 lds_write16(smem, off, v);
             } else {
                 u32x2 v;
-                v.x = r[a][0]; v.y = r[a][1];
+                v.x = r[2 * a + 0]; v.y = r[2 * a + 1];
                 lds_write8(smem, off, v);
             }
         }
     }
-    __device__ __forceinline__ void store(char* smem, int tid) const {
+    static __device__ __forceinline__ void store(const uint32_t (&r)[StageRegs<D>::kCount], char* smem, int tid) {
         const int rq = row_quad(tid), c = col_chunk(tid);
 #pragma unroll
         for (int wd = 0; wd < kWords; ++wd) {
             // even column: low halves of the four rows; odd column: high halves
             u32x2 ev, od;
-            ev.x = __builtin_amdgcn_perm(r[1][wd], r[0][wd], 0x05040100u);
-            ev.y = __builtin_amdgcn_perm(r[3][wd], r[2][wd], 0x05040100u);
-            od.x = __builtin_amdgcn_perm(r[1][wd], r[0][wd], 0x07060302u);
-            od.y = __builtin_amdgcn_perm(r[3][wd], r[2][wd], 0x07060302u);
+            ev.x = __builtin_amdgcn_perm(r[1 * kWords + wd], r[0 * kWords + wd], 0x05040100u);
+            ev.y = __builtin_amdgcn_perm(r[3 * kWords + wd], r[2 * kWords + wd], 0x05040100u);
+            od.x = __builtin_amdgcn_perm(r[1 * kWords + wd], r[0 * kWords + wd], 0x07060302u);
+            od.y = __builtin_amdgcn_perm(r[3 * kWords + wd], r[2 * kWords + wd], 0x07060302u);
             const int d = c * kCols + 2 * wd;
             lds_write8(smem, TransTile::write_off(d, rq), ev);
             lds_write8(smem, TransTile::write_off(d + 1, rq), od);
@@ -216,20 +228,34 @@ struct TransStage {
 };
 
 // Workgroup -> (head, tile) mapping. Workgroups are dealt round-robin to the 8 XCDs, each with
-// its own L2: give every XCD whole heads, walk the tiles of a head consecutively so its K/V
-// stay in that L2, and start with the heaviest tiles (highest index first when `reverse`).
-__device__ __forceinline__ void map_block(int bid, int num_heads, int num_tiles, bool reverse, int* bh, int* tile) {
+// its own L2, so every XCD is given whole heads (head % 8 == XCD). With uniform tiles the XCD
+// walks head after head, which keeps one head's K/V in its L2. With causal tiles (work grows or
+// shrinks with the tile index) it instead walks tile by tile from the heaviest down, all of
+// its heads abreast: a dispatcher that hands the next workgroup to the first free slot then pairs
+// long and short workgroups (longest-processing-time order), and workgroups of one head that
+// start together stream the same K/V tiles at the same time.
+enum TileOrder { kUniformTiles = 0, kHeavyLast = 1, kHeavyFirst = 2 };
+__device__ __forceinline__ void map_block(int bid, int num_heads, int num_tiles, int order, int* bh, int* tile) {
     int head, t;
+    const bool heavy_last = order == kHeavyLast;
     if ((num_heads & 7) == 0) {
-        const int xcd = bid & 7, slot = bid >> 3;
-        head = (slot / num_tiles) * 8 + xcd;
-        t = slot % num_tiles;
+        const int xcd = bid & 7, slot = bid >> 3, heads_per_xcd = num_heads >> 3;
+        if (order != kUniformTiles) {
+            head = (slot % heads_per_xcd) * 8 + xcd;
+            t = slot / heads_per_xcd;
+        } else {
+            head = (slot / num_tiles) * 8 + xcd;
+            t = slot % num_tiles;
+        }
+    } else if (order != kUniformTiles) {
+        head = bid % num_heads;
+        t = bid / num_heads;
     } else {
         head = bid / num_tiles;
         t = bid % num_tiles;
     }
     *bh = head;
-    *tile = reverse ? num_tiles - 1 - t : t;
+    *tile = heavy_last ? num_tiles - 1 - t : t;
 }
 
 // Dropout bytes for 4 consecutive columns j0..j0+3 (j0 % 4 == 0) of row i: one 32-bit word.

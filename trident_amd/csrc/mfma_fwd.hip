@@ -1,37 +1,50 @@
 // Forward attention on the matrix cores: online-softmax flash kernel for fp16/bf16,
 // D in {64,128}, S a multiple of 128 (replaces trident/kernel/attention.py:33-165).
 //
-// One workgroup (4 waves) owns 128 query rows, one wave 32 of them. Q stays in registers as
-// the B operand of S^T = K Q^T; K (row-major, padded) and V^T (transposed, slot-permuted)
-// tiles of 64 keys are double-buffered in LDS and filled with 16-byte global loads issued one
-// tile ahead. S^T and O^T = V^T P^T accumulate in fp32; P goes from the S^T accumulators to
-// the B operand of the second MFMA in registers. The row statistics live one per lane; the
-// two lane halves of a row are combined with one cross-lane exchange per tile.
+// A workgroup of NW waves owns 32*NW query rows, one wave 32 of them. Q stays in registers as
+// the B operand of S^T = K Q^T; K (row-major, padded) and V^T (transposed, slot-permuted) tiles
+// of 64 keys live in a three-stage LDS ring that is filled through registers one tile ahead of
+// its use and loaded from HBM two tiles ahead. S^T and O^T = V^T P^T accumulate in fp32; P goes
+// from the S^T accumulators to the B operand of the second MFMA in registers. The row
+// statistics live one per lane; the two lane halves of a row are combined with one cross-lane
+// exchange per tile.
+//
+// With 8 waves (two per SIMD) the upper four run one half-step behind the lower four: they
+// multiply the previous tile's P with V before they compute the scores of the current tile, so
+// while one wave of a SIMD is in its softmax (vector ALU) the other one feeds the matrix pipe.
 #include "launch.hpp"
 #include "mfma_common.hpp"
 
 namespace tri {
 namespace {
 
-constexpr int kBM = 128;  // query rows per workgroup
-constexpr int kBN = 64;   // keys per tile
+constexpr int kBN = 64;      // keys per tile
+constexpr int kStages = 3;   // LDS ring depth
 constexpr float kTau = 8.f;  // lazy-rescale threshold, log2 domain
 
 enum MaskKind { kNoMask = 0, kMaskF32 = 1, kMaskT = 2 };
 
-template <typename T, int D, bool CAUSAL, int MASK, bool DROPOUT>
-__global__ __launch_bounds__(256, 2) void mfma_fwd_kernel(const KParams p) {
+template <typename T, int D, int NW, bool CAUSAL, int MASK, bool DROPOUT>
+__global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
+    constexpr int kBM = 32 * NW;
     constexpr int kKBytes = RowTile<D>::bytes(kBN);
     constexpr int kVBytes = TransTile::bytes(D);
     constexpr int kStageBytes = kKBytes + kVBytes;
     constexpr int KK = D / 16;  // K-steps of S^T
     constexpr int DB = D / 32;  // 32-row blocks of O^T
-    __shared__ __attribute__((aligned(16))) char smem[2 * kStageBytes];
+    constexpr int kSteps = 2 * KK, kAhead = 8;
+    constexpr int kPvSteps = 4 * DB, kPvAhead = 8;
+    __shared__ __attribute__((aligned(16))) char smem[kStages * kStageBytes];
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+    const int ltid = tid & 255;                    // index within the 256 threads that stage one matrix
+    const bool skew = NW == 8 && wave >= 4;        // runs P V one tile late
+    const bool stage_v = NW == 4 || wave < 4;      // which matrix this wave moves HBM -> LDS
+    const bool stage_k = NW == 4 || wave >= 4;
     int bh, qt;
-    map_block(blockIdx.x, p.B * p.H, p.S / kBM, true, &bh, &qt);
+    map_block(blockIdx.x, p.B * p.H, p.S / kBM, CAUSAL ? kHeavyLast : kUniformTiles, &bh, &qt);
     const int b = bh / p.H, hd = bh % p.H;
     const int q0 = qt * kBM;
     const int wrow0 = q0 + 32 * wave;  // first query row of this wave
@@ -50,36 +63,65 @@ __global__ __launch_bounds__(256, 2) void mfma_fwd_kernel(const KParams p) {
     f32x16 oacc[DB];
 #pragma unroll
     for (int db = 0; db < DB; ++db) oacc[db] = zero16();
-    float m = -INFINITY, l = 0.f;  // running max (log2 domain, scaled) and this lane's partial sum
+    float m = -INFINITY, l = 0.f;  // reference exponent (log2 domain, scaled) and this lane's partial sum
 
-    const int n_tiles = CAUSAL ? (q0 + kBM) / kBN : p.S / kBN;
+    const int n_tiles = CAUSAL ? (q0 + kBM) / kBN : p.S / kBN;            // tiles the workgroup streams
+    const int my_tiles = CAUSAL ? (wrow0 + 31) / kBN + 1 : n_tiles;       // tiles this wave has visible keys in
     const float c = p.scale_log2;
 
-    RowStage<D> kst;
-    TransStage<T, D> vst;
-    kst.load(kbase, krow_bytes, tid);
-    vst.load(vbase, vrow_bytes, tid);
-    kst.store(smem, tid);
-    vst.store(smem + kKBytes, tid);
-    // every global load issued so far (Q fragments, first tile) has landed: without this the
-    // compiler keeps waiting on vmcnt inside the loop and serialises each tile's prefetch
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    // staging registers: with 8 waves a wave moves either K or V and one buffer serves both roles
+    uint32_t sreg[StageRegs<D>::kCount];
+    uint32_t sreg2[NW == 4 ? StageRegs<D>::kCount : 1];
+    if (stage_k) {
+        RowStage<D>::load(sreg, kbase, krow_bytes, ltid);
+        RowStage<D>::store(sreg, smem, ltid);
+        if (n_tiles > 1) RowStage<D>::load(sreg, kbase + kBN * krow_bytes, krow_bytes, ltid);
+    }
+    if constexpr (NW == 4) {
+        TransStage<D>::load(sreg2, vbase, vrow_bytes, ltid);
+        TransStage<D>::store(sreg2, smem + kKBytes, ltid);
+        if (n_tiles > 1) TransStage<D>::load(sreg2, vbase + kBN * vrow_bytes, vrow_bytes, ltid);
+    } else if (stage_v) {
+        TransStage<D>::load(sreg, vbase, vrow_bytes, ltid);
+        TransStage<D>::store(sreg, smem + kKBytes, ltid);
+        if (n_tiles > 1) TransStage<D>::load(sreg, vbase + kBN * vrow_bytes, vrow_bytes, ltid);
+    }
     __syncthreads();
 
-    for (int j = 0; j < n_tiles; ++j) {
-        const char* sK = smem + (j & 1) * kStageBytes;
+    u32x4 pb[4];  // P of the current tile as four B operands (kept across the step by skewed waves)
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) pb[ks] = u32x4{0, 0, 0, 0};
+
+    const int n_iter = NW == 8 ? n_tiles + 1 : n_tiles;
+    for (int j = 0; j < n_iter; ++j) {
+        const char* sK = smem + (j % kStages) * kStageBytes;
         const char* sV = sK + kKBytes;
         const int t0 = j * kBN;
-        const bool more = j + 1 < n_tiles;
-        if (more) {
-            kst.load(kbase + (t0 + kBN) * krow_bytes, krow_bytes, tid);
-            vst.load(vbase + (t0 + kBN) * vrow_bytes, vrow_bytes, tid);
+
+        // ---- skewed waves: O^T += V^T P^T of the previous tile
+        if (skew && j >= 1 && j - 1 < my_tiles) {
+            const char* pV = smem + ((j - 1) % kStages) * kStageBytes + kKBytes;
+            u32x4 vring[kPvAhead];
+#pragma unroll
+            for (int s = 0; s < kPvAhead; ++s)
+                vring[s] = lds_read16(pV, TransTile::read_off(32 * (s % DB) + l32, s / DB, h));
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s = 0; s < kPvSteps; ++s) {
+                oacc[s % DB] = Mma<T>::run(vring[s % kPvAhead], pb[s / DB], oacc[s % DB]);
+                if (s + kPvAhead < kPvSteps) {
+                    const int n = s + kPvAhead;
+                    vring[s % kPvAhead] = lds_read16(pV, TransTile::read_off(32 * (n % DB) + l32, n / DB, h));
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
-        const bool active = !CAUSAL || t0 <= wrow0 + 31;
+
+        const bool active = j < my_tiles;
+        float x[32];  // scores of this lane: x[16*kb + i] is key t0 + 32*kb + c_row(i,h)
+        float mk[MASK != kNoMask ? 32 : 1];
         if (active) {
-            float x[32];  // scores of this lane: x[16*kb + i] is key t0 + 32*kb + c_row(i,h)
             // additive mask for this lane's row: issued before the MFMAs, used after them
-            float mk[MASK != kNoMask ? 32 : 1];
             if constexpr (MASK != kNoMask) {
                 const int64_t mrow = b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(qrow) * p.ms[2] + t0;
 #pragma unroll
@@ -95,38 +137,46 @@ __global__ __launch_bounds__(256, 2) void mfma_fwd_kernel(const KParams p) {
                     }
                 }
             }
-            // S^T = K Q^T with the A fragments requested kAhead MFMAs before their use, so that
-            // the LDS latency overlaps the matrix pipe instead of stalling every MFMA pair
-            {
-                constexpr int kSteps = 2 * KK, kAhead = 8;
-                u32x4 ring[kAhead];
+            // S^T = K Q^T with the A fragments requested kAhead MFMAs before their use
+            u32x4 ring[kAhead];
 #pragma unroll
-                for (int s = 0; s < kAhead; ++s)
-                    ring[s] = lds_read16(sK, RowTile<D>::off(32 * (s / KK) + l32, 2 * (s % KK) + h));
-                __builtin_amdgcn_sched_barrier(0);
-                f32x16 st[2] = {zero16(), zero16()};
-#pragma unroll
-                for (int s = 0; s < kSteps; ++s) {
-                    st[s / KK] = Mma<T>::run(ring[s % kAhead], qf[s % KK], st[s / KK]);
-                    if (s + kAhead < kSteps) {
-                        const int n = s + kAhead;
-                        ring[s % kAhead] = lds_read16(sK, RowTile<D>::off(32 * (n / KK) + l32, 2 * (n % KK) + h));
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    x[i] = st[0][i];
-                    x[16 + i] = st[1][i];
-                }
-            }
-            // first V^T fragments of the second product: requested now, they arrive during the softmax
-            constexpr int kPvSteps = 4 * DB, kPvAhead = 8;
-            u32x4 vring[kPvAhead];
-#pragma unroll
-            for (int s = 0; s < kPvAhead; ++s)
-                vring[s] = lds_read16(sV, TransTile::read_off(32 * (s % DB) + l32, s / DB, h));
+            for (int s = 0; s < kAhead; ++s)
+                ring[s] = lds_read16(sK, RowTile<D>::off(32 * (s / KK) + l32, 2 * (s % KK) + h));
             __builtin_amdgcn_sched_barrier(0);
+            f32x16 st[2] = {zero16(), zero16()};
+#pragma unroll
+            for (int s = 0; s < kSteps; ++s) {
+                st[s / KK] = Mma<T>::run(ring[s % kAhead], qf[s % KK], st[s / KK]);
+                if (s + kAhead < kSteps) {
+                    const int n = s + kAhead;
+                    ring[s % kAhead] = lds_read16(sK, RowTile<D>::off(32 * (n / KK) + l32, 2 * (n % KK) + h));
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                x[i] = st[0][i];
+                x[16 + i] = st[1][i];
+            }
+        }
+
+        // ---- staging: tile j+1 registers -> LDS, tile j+2 HBM -> registers (runs under the MFMAs)
+        if (j + 1 < n_tiles) {
+            char* nK = smem + ((j + 1) % kStages) * kStageBytes;
+            if (stage_k) {
+                RowStage<D>::store(sreg, nK, ltid);
+                if (j + 2 < n_tiles) RowStage<D>::load(sreg, kbase + (t0 + 2 * kBN) * krow_bytes, krow_bytes, ltid);
+            }
+            if constexpr (NW == 4) {
+                TransStage<D>::store(sreg2, nK + kKBytes, ltid);
+                if (j + 2 < n_tiles) TransStage<D>::load(sreg2, vbase + (t0 + 2 * kBN) * vrow_bytes, vrow_bytes, ltid);
+            } else if (stage_v) {
+                TransStage<D>::store(sreg, nK + kKBytes, ltid);
+                if (j + 2 < n_tiles) TransStage<D>::load(sreg, vbase + (t0 + 2 * kBN) * vrow_bytes, vrow_bytes, ltid);
+            }
+        }
+
+        if (active) {
             // scores in the log2 domain; without a mask the scale is folded into the exponent
             if constexpr (MASK != kNoMask) {
 #pragma unroll
@@ -179,9 +229,8 @@ __global__ __launch_bounds__(256, 2) void mfma_fwd_kernel(const KParams p) {
                     }
                 }
             }
-            // O^T += V^T P^T; without dropout the row sum is taken from the rounded P that is
+            // P as B operands; without dropout the row sum is taken from the rounded P that is
             // actually multiplied with V, two values per instruction
-            u32x4 pb[4];
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) {
                 pb[ks] = pack8<T>(&x[8 * ks]);
@@ -192,22 +241,24 @@ __global__ __launch_bounds__(256, 2) void mfma_fwd_kernel(const KParams p) {
                     psum = Mma<T>::add_pair(pb[ks].w, psum);
                 }
             }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int s = 0; s < kPvSteps; ++s) {
-                oacc[s % DB] = Mma<T>::run(vring[s % kPvAhead], pb[s / DB], oacc[s % DB]);
-                if (s + kPvAhead < kPvSteps) {
-                    const int n = s + kPvAhead;
-                    vring[s % kPvAhead] = lds_read16(sV, TransTile::read_off(32 * (n % DB) + l32, n / DB, h));
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
             l += psum;
-        }
-        if (more) {
-            char* nK = smem + ((j + 1) & 1) * kStageBytes;
-            kst.store(nK, tid);
-            vst.store(nK + kKBytes, tid);
+            // non-skewed waves: O^T += V^T P^T now
+            if (!skew) {
+                u32x4 vring[kPvAhead];
+#pragma unroll
+                for (int s = 0; s < kPvAhead; ++s)
+                    vring[s] = lds_read16(sV, TransTile::read_off(32 * (s % DB) + l32, s / DB, h));
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int s = 0; s < kPvSteps; ++s) {
+                    oacc[s % DB] = Mma<T>::run(vring[s % kPvAhead], pb[s / DB], oacc[s % DB]);
+                    if (s + kPvAhead < kPvSteps) {
+                        const int n = s + kPvAhead;
+                        vring[s % kPvAhead] = lds_read16(sV, TransTile::read_off(32 * (n % DB) + l32, n / DB, h));
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
         }
         __syncthreads();
     }
@@ -227,29 +278,36 @@ __global__ __launch_bounds__(256, 2) void mfma_fwd_kernel(const KParams p) {
     if (h == 0) p.lse[static_cast<int64_t>(bh) * p.S + qrow] = m + fast_log2(l);
 }
 
-template <typename T, int D, bool CAUSAL, int MASK>
+template <typename T, int D, int NW, bool CAUSAL, int MASK>
 int launch_fwd_dropout(const KParams& p, hipStream_t stream) {
-    const dim3 grid(p.B * p.H * (p.S / kBM)), block(256);
-    if (p.thr8 > 0) hipLaunchKernelGGL((mfma_fwd_kernel<T, D, CAUSAL, MASK, true>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((mfma_fwd_kernel<T, D, CAUSAL, MASK, false>), grid, block, 0, stream, p);
+    const dim3 grid(p.B * p.H * (p.S / (32 * NW))), block(64 * NW);
+    if (p.thr8 > 0) hipLaunchKernelGGL((mfma_fwd_kernel<T, D, NW, CAUSAL, MASK, true>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((mfma_fwd_kernel<T, D, NW, CAUSAL, MASK, false>), grid, block, 0, stream, p);
     return static_cast<int>(hipGetLastError());
 }
 
-template <typename T, int D>
+template <typename T, int D, int NW>
 int launch_fwd_variant(int dtype, const KParams& p, hipStream_t stream) {
-    if (p.causal) return launch_fwd_dropout<T, D, true, kNoMask>(p, stream);
-    if (p.mask == nullptr) return launch_fwd_dropout<T, D, false, kNoMask>(p, stream);
-    if (p.mask_dtype == TRI_ATTN_F32) return launch_fwd_dropout<T, D, false, kMaskF32>(p, stream);
-    if (p.mask_dtype == dtype) return launch_fwd_dropout<T, D, false, kMaskT>(p, stream);
+    if (p.causal) return launch_fwd_dropout<T, D, NW, true, kNoMask>(p, stream);
+    if (p.mask == nullptr) return launch_fwd_dropout<T, D, NW, false, kNoMask>(p, stream);
+    if (p.mask_dtype == TRI_ATTN_F32) return launch_fwd_dropout<T, D, NW, false, kMaskF32>(p, stream);
+    if (p.mask_dtype == dtype) return launch_fwd_dropout<T, D, NW, false, kMaskT>(p, stream);
     return TRI_ATTN_EDTYPE;
+}
+
+template <typename T, int D>
+int launch_fwd_waves(int dtype, const KParams& p, hipStream_t stream) {
+    // 8 waves (256 query rows) when the sequence allows it: two waves per SIMD out of phase
+    if (p.S % 256 == 0) return launch_fwd_variant<T, D, 8>(dtype, p, stream);
+    return launch_fwd_variant<T, D, 4>(dtype, p, stream);
 }
 
 }  // namespace
 
 int launch_mfma_fwd(int dtype, const KParams& p, hipStream_t stream) {
     if (dtype == TRI_ATTN_BF16)
-        return p.D == 128 ? launch_fwd_variant<bf16_t, 128>(dtype, p, stream) : launch_fwd_variant<bf16_t, 64>(dtype, p, stream);
-    return p.D == 128 ? launch_fwd_variant<f16_t, 128>(dtype, p, stream) : launch_fwd_variant<f16_t, 64>(dtype, p, stream);
+        return p.D == 128 ? launch_fwd_waves<bf16_t, 128>(dtype, p, stream) : launch_fwd_waves<bf16_t, 64>(dtype, p, stream);
+    return p.D == 128 ? launch_fwd_waves<f16_t, 128>(dtype, p, stream) : launch_fwd_waves<f16_t, 64>(dtype, p, stream);
 }
 
 }  // namespace tri
