@@ -316,17 +316,29 @@ __global__ __launch_bounds__(256, 2) void mfma_dkdv_kernel(const KParams p) {
 }
 
 // ---------------------------------------------------------------------------------- launch
+template <typename T, int D, bool CAUSAL, int MASK>
+int launch_dq_dropout(const KParams& p, hipStream_t stream) {
+    const dim3 grid(p.B * p.H * (p.S / kBM)), block(256);
+    if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dq_kernel<T, D, CAUSAL, MASK, true>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((mfma_dq_kernel<T, D, CAUSAL, MASK, false>), grid, block, 0, stream, p);
+    return static_cast<int>(hipGetLastError());
+}
+
+template <typename T, int D, bool CAUSAL, int MASK>
+int launch_dkdv_dropout(const KParams& p, hipStream_t stream) {
+    const dim3 grid(p.B * p.H * (p.S / kBM)), block(256);
+    if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, CAUSAL, MASK, true>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, CAUSAL, MASK, false>), grid, block, 0, stream, p);
+    return static_cast<int>(hipGetLastError());
+}
+
 template <int WHICH, typename T, int D, bool CAUSAL, int MASK>
 int launch_bwd_dropout(const KParams& p, hipStream_t stream) {
-    const dim3 grid(p.B * p.H * (p.S / kBM)), block(256);
-    if (WHICH == kMfmaDq) {
-        if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dq_kernel<T, D, CAUSAL, MASK, true>), grid, block, 0, stream, p);
-        else hipLaunchKernelGGL((mfma_dq_kernel<T, D, CAUSAL, MASK, false>), grid, block, 0, stream, p);
+    if constexpr (WHICH == kMfmaDq) {
+        return launch_dq_dropout<T, D, CAUSAL, MASK>(p, stream);
     } else {
-        if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, CAUSAL, MASK, true>), grid, block, 0, stream, p);
-        else hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, CAUSAL, MASK, false>), grid, block, 0, stream, p);
+        return launch_dkdv_dropout<T, D, CAUSAL, MASK>(p, stream);
     }
-    return static_cast<int>(hipGetLastError());
 }
 
 template <int WHICH, typename T, int D>

@@ -128,6 +128,67 @@ __device__ __forceinline__ u32x4 lds_read16(const char* smem, int off) {
 __device__ __forceinline__ void lds_write16(char* smem, int off, u32x4 v) { *reinterpret_cast<u32x4*>(smem + off) = v; }
 __device__ __forceinline__ void lds_write8(char* smem, int off, u32x2 v) { *reinterpret_cast<u32x2*>(smem + off) = v; }
 
+// ---------------------------------------------------------------- swizzled tiles filled by LDS-direct loads
+// Row-major tile [64][D] of 16-bit elements without padding, filled straight from HBM with
+// global_load_lds_dwordx4 (no registers, no ds_write): one wave instruction deposits 64 x 16
+// bytes at consecutive LDS addresses, so a lane can only choose WHICH 16-byte chunk of its row it
+// fetches, and the bank-conflict-free layout is an XOR swizzle of the chunk index with the row.
+// Both operand forms are read from the same tile:
+//   row fragment   A[M = tile row][K = column]: one ds_read_b128 (rows r..r+31, chunk 2kk+h)
+//   transposed     A[M = column][K = tile row]: two ds_read_b64_tr_b16; in each 16-lane group
+//                  lane i receives the element (column base + i) of 4 consecutive tile rows
+//                  when lane j points at row (base + j/4), columns 4*(j%4) .. +3.
+// The transposed form yields the K-slot order of the C registers (see the top of this file)
+// without any permuted storage.
+#define TRI_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+#define TRI_GLB_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+template <int D>
+struct SwzTile {
+    static constexpr int kRowBytes = D * 2;
+    static constexpr int kChunks = D / 8;               // 16-byte chunks per row
+    static constexpr int kBytes = 64 * kRowBytes;       // 16 KiB (D=128) or 8 KiB (D=64)
+    static constexpr int kBlocks = kBytes / 1024;       // wave instructions per tile
+    static constexpr int kRowsPerBlock = 1024 / kRowBytes;
+    // chunk swizzle: 16 consecutive rows (b128 reads) and 4 consecutive rows x 32 bytes (tr reads)
+    // land in distinct banks
+    static __device__ __forceinline__ int swz(int r) {
+        if constexpr (D == 128) return ((r & 7) << 1) | ((r >> 3) & 1);
+        else return (((r >> 1) & 3) << 1) | ((r >> 3) & 1);
+    }
+    static __device__ __forceinline__ int off(int r, int c) { return r * kRowBytes + ((c ^ swz(r)) << 4); }
+
+    // Per-lane source offset (bytes from the tile's first row) of block `blk` (0..kBlocks-1).
+    static __device__ __forceinline__ int64_t src_off(int blk, int lane, int64_t row_stride_bytes) {
+        const int row = blk * kRowsPerBlock + lane / kChunks;
+        const int c = (lane % kChunks) ^ swz(row);
+        return row * row_stride_bytes + c * 16;
+    }
+    static __device__ __forceinline__ void load_block(char* tile, int blk, const char* src) {
+        __builtin_amdgcn_global_load_lds(TRI_GLB_PTR(src), TRI_LDS_PTR(tile + blk * 1024), 16, 0, 0);
+    }
+    // byte offset (within the tile) a lane passes to the transposed read of column block db
+    // (32 columns), half = 0/1 (K-slots 0-3 / 4-7); add ks * 16 * kRowBytes for K-step ks
+    static __device__ __forceinline__ int tr_off(int db, int half, int lane) {
+        const int g = lane >> 4, lam = lane & 15;
+        const int r = 8 * half + 4 * (g >> 1) + (lam >> 2);
+        const int col = 32 * db + 16 * (g & 1) + 4 * (lam & 3);
+        return r * kRowBytes + (((col >> 3) ^ swz(r)) << 4) + ((lam & 1) << 3);
+    }
+    static __device__ __forceinline__ u32x4 tr_frag(const char* tile, int off_half0, int off_half1, int ks) {
+        const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) s16x4*)(tile + off_half0 + ks * 16 * kRowBytes));
+        const s16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) s16x4*)(tile + off_half1 + ks * 16 * kRowBytes));
+        u32x2 lo = __builtin_bit_cast(u32x2, a), hi = __builtin_bit_cast(u32x2, b);
+        return u32x4{lo.x, lo.y, hi.x, hi.y};
+    }
+};
+
+// s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14)
+#define TRI_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
+
 // ---------------------------------------------------------------- HBM -> registers -> LDS staging
 // One [64][D] tile of 16-bit elements is moved by 256 threads, D/8 registers each. Both layouts
 // below work on the same raw register array, so a wave that stages K and a wave that stages V
