@@ -25,7 +25,13 @@ HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (see profiles/); None where not measured.
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {
+    # (workload, kernel): bytes read + written per launch (profiles/c3_hbm_traffic.txt)
+    ("C3", "fwd"): int((155.6 + 34.5) * 2**20),
+    ("C3", "bwd_dkdv"): int((210.6 + 64.0) * 2**20),
+    ("C3", "bwd_dq"): int((705.5 + 78.0) * 2**20),
+    ("C3", "bwd_delta"): int((64.0 + 0.5) * 2**20),
+}
 
 
 def _dtype_name(dtype):
@@ -161,6 +167,9 @@ def main():
     ap.add_argument("--workload", default="C3")
     ap.add_argument("--report", action="store_true", help="also print all five configurations on stderr")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy (known HBM traffic) so that rocprofv3 FETCH_SIZE / "
+                         "WRITE_SIZE readings of the attention kernels can be scaled against it")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build runs on one GPU; the attention path has no exchange step to "
@@ -174,6 +183,13 @@ def main():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
     w = workloads.WORKLOADS[a.workload]
+    if a.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     path = Path(w, dev)
     wall_ms, per_kernel = run_steps(path, a.steps, a.warmup)
     dname = _dtype_name(w.dtype)
