@@ -28,23 +28,31 @@ __device__ __forceinline__ float mask_at(const void* mask, int64_t off) {
 }
 
 // ------------------------------------------------------------------------------------ dQ
-template <typename T, int D, bool CAUSAL, int MASK, bool DROPOUT>
-__global__ __launch_bounds__(256, 2) void mfma_dq_kernel(const KParams p) {
-    constexpr int kRowBytes = RowTile<D>::bytes(kBN);
-    constexpr int kTransBytes = TransTile::bytes(D);
+// A workgroup of NW waves owns 32*NW query rows, one wave 32 of them with its Q and dO rows in
+// registers (B operands) and dQ^T in fp32 accumulators; two waves per SIMD. K and V stream as
+// 64-key swizzled LDS tiles in a ring of 4, filled by LDS-direct loads three tiles ahead (no
+// staging registers, no ds_write). Per 32-key block: S^T = K Q^T and dP^T = V dO^T from row
+// fragments, dS^T = P^T (dP^T - delta) on the vector ALU, dQ^T += K^T dS^T with K^T read through
+// transposed LDS reads of the same K tile.
+template <typename T, int D, int NW, bool CAUSAL, int MASK, bool DROPOUT>
+__global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
+    using Tile = SwzTile<D>;
+    constexpr int kRows = 32 * NW;
+    constexpr int kStages = 4;
+    constexpr int kStageBytes = 2 * Tile::kBytes;  // K tile, V tile
     constexpr int KK = D / 16;
     constexpr int DB = D / 32;
-    __shared__ __attribute__((aligned(16))) char smem[2 * kRowBytes + kTransBytes];
-    char* sK = smem;
-    char* sV = smem + kRowBytes;
-    char* sKt = smem + 2 * kRowBytes;
+    constexpr int kBlocksPerWave = 2 * Tile::kBlocks / NW;  // LDS-direct loads per wave and tile
+    static_assert(2 * Tile::kBlocks % NW == 0, "tile blocks must divide among the waves");
+    __shared__ __attribute__((aligned(1024))) char smem[kStages * kStageBytes];
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63, l32 = lane & 31, h = lane >> 5;
     int bh, qt;
-    map_block(blockIdx.x, p.B * p.H, p.S / kBM, CAUSAL ? kHeavyLast : kUniformTiles, &bh, &qt);
+    map_block(blockIdx.x, p.B * p.H, p.S / kRows, CAUSAL ? kHeavyLast : kUniformTiles, &bh, &qt);
     const int b = bh / p.H, hd = bh % p.H;
-    const int q0 = qt * kBM;
+    const int q0 = qt * kRows;
     const int wrow0 = q0 + 32 * wave;
     const int qrow = wrow0 + l32;
 
@@ -69,80 +77,107 @@ __global__ __launch_bounds__(256, 2) void mfma_dq_kernel(const KParams p) {
 #pragma unroll
     for (int db = 0; db < DB; ++db) acc[db] = zero16();
 
-    const int n_tiles = CAUSAL ? (q0 + kBM) / kBN : p.S / kBN;
-    uint32_t kst[StageRegs<D>::kCount], vst[StageRegs<D>::kCount];
-    TransStage<D>::load(kst, kbase, krow_bytes, tid);
-    RowStage<D>::load(vst, vbase, vrow_bytes, tid);
-    // all loads issued so far have landed; otherwise the compiler waits on vmcnt in the loop
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    const int n_tiles = CAUSAL ? (q0 + kRows) / kBN : p.S / kBN;        // tiles the workgroup streams
+    const int my_tiles = CAUSAL ? (wrow0 + 31) / kBN + 1 : n_tiles;     // tiles with keys visible to this wave
+
+    int src_off[kBlocksPerWave];
+#pragma unroll
+    for (int i = 0; i < kBlocksPerWave; ++i) {
+        const int blk = wave * kBlocksPerWave + i;  // 0 .. 2*kBlocks-1 over the K tile then the V tile
+        const bool is_v = blk >= Tile::kBlocks;
+        src_off[i] = static_cast<int>(Tile::src_off(is_v ? blk - Tile::kBlocks : blk, lane, is_v ? vrow_bytes : krow_bytes));
+    }
+    auto issue_tile = [&](int t) {
+        char* stage = smem + (t % kStages) * kStageBytes;
+#pragma unroll
+        for (int i = 0; i < kBlocksPerWave; ++i) {
+            const int blk = wave * kBlocksPerWave + i;
+            const bool is_v = blk >= Tile::kBlocks;
+            const char* tile_src = is_v ? vbase + static_cast<int64_t>(t) * kBN * vrow_bytes
+                                        : kbase + static_cast<int64_t>(t) * kBN * krow_bytes;
+            __builtin_amdgcn_global_load_lds(TRI_GLB_PTR(tile_src + src_off[i]), TRI_LDS_PTR(stage + blk * 1024), 16, 0, 0);
+        }
+    };
+    issue_tile(0);
+    if (1 < n_tiles) issue_tile(1);
+    if (2 < n_tiles) issue_tile(2);
+
+    const int row_off0 = Tile::off(l32, h);
+    const int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
 
     for (int j = 0; j < n_tiles; ++j) {
-        const int t0 = j * kBN;
-        TransStage<D>::store_rows(kst, sK, tid);
-        TransStage<D>::store(kst, sKt, tid);
-        RowStage<D>::store(vst, sV, tid);
-        __syncthreads();
-        if (j + 1 < n_tiles) {
-            TransStage<D>::load(kst, kbase + (t0 + kBN) * krow_bytes, krow_bytes, tid);
-            RowStage<D>::load(vst, vbase + (t0 + kBN) * vrow_bytes, vrow_bytes, tid);
+        // tile j has landed (up to two younger tiles may still be in flight) and is visible to all
+        // waves; every wave is done with tile j-1, whose slot takes the load of tile j+3
+        {
+            const int younger = min(2, n_tiles - 1 - j);
+            if (younger == 2) TRI_WAIT_VMCNT(2 * kBlocksPerWave);
+            else if (younger == 1) TRI_WAIT_VMCNT(kBlocksPerWave);
+            else TRI_WAIT_VMCNT(0);
         }
-        const bool active = !CAUSAL || t0 <= wrow0 + 31;
-        if (active) {
-            const bool diag = CAUSAL && t0 + kBN - 1 > wrow0;
+        __syncthreads();
+        if (j + 3 < n_tiles) issue_tile(j + 3);
+        if (j >= my_tiles) continue;
+
+        const char* sK = smem + (j % kStages) * kStageBytes;
+        const char* sV = sK + Tile::kBytes;
+        const int t0 = j * kBN;
+        const bool diag = CAUSAL && t0 + kBN - 1 > wrow0;
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                float mk[MASK != kNoMask ? 16 : 1];
-                if constexpr (MASK != kNoMask) {
-                    const int64_t mrow = b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(qrow) * p.ms[2] + t0 + 32 * kb;
+        for (int kb = 0; kb < 2; ++kb) {
+            float mk[MASK != kNoMask ? 16 : 1];
+            if constexpr (MASK != kNoMask) {
+                const int64_t mrow = b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(qrow) * p.ms[2] + t0 + 32 * kb;
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) mk[i] = mask_at<T, MASK>(p.mask, mrow + c_row(i, h));
-                }
-                f32x16 st = zero16(), dpt = zero16();
+                for (int i = 0; i < 16; ++i) mk[i] = mask_at<T, MASK>(p.mask, mrow + c_row(i, h));
+            }
+            u32x4 fr[KK];
 #pragma unroll
-                for (int kk = 0; kk < KK; ++kk) {
-                    const u32x4 a = lds_read16(sK, RowTile<D>::off(32 * kb + l32, 2 * kk + h));
-                    st = Mma<T>::run(a, qf[kk], st);
-                }
+            for (int kk = 0; kk < KK; ++kk) fr[kk] = lds_read16(sK, (row_off0 ^ (kk << 5)) + 32 * kb * Tile::kRowBytes);
+            __builtin_amdgcn_sched_barrier(0);
+            f32x16 st = zero16(), dpt = zero16();
 #pragma unroll
-                for (int kk = 0; kk < KK; ++kk) {
-                    const u32x4 a = lds_read16(sV, RowTile<D>::off(32 * kb + l32, 2 * kk + h));
-                    dpt = Mma<T>::run(a, gf[kk], dpt);
-                }
-                float ds[16];
+            for (int kk = 0; kk < KK; ++kk) {
+                st = Mma<T>::run(fr[kk], qf[kk], st);
+                fr[kk] = lds_read16(sV, (row_off0 ^ (kk << 5)) + 32 * kb * Tile::kRowBytes);
+                __builtin_amdgcn_sched_barrier(0);
+            }
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int key = t0 + 32 * kb + c_row(i, h);
-                    float x = st[i] * c;
-                    if constexpr (MASK != kNoMask) x = fmaf(mk[i], kLog2e, x);
-                    float pr = fast_exp2(x - lse);
-                    if (diag) pr = key <= qrow ? pr : 0.f;
-                    ds[i] = pr;
-                }
-                if constexpr (DROPOUT) {
+            for (int kk = 0; kk < KK; ++kk) dpt = Mma<T>::run(fr[kk], gf[kk], dpt);
+            // first transposed K fragments of this block: they arrive during the vector-ALU part
+            u32x4 tf[2 * DB];
 #pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const uint32_t w = dropout_word(p, bh, qrow, t0 + 32 * kb + 8 * g + 4 * h);
+            for (int i = 0; i < 2 * DB; ++i)
+                tf[i] = Tile::tr_frag(sK, tr_off0 ^ ((i % DB) << 6), tr_off1 ^ ((i % DB) << 6), 2 * kb + i / DB);
+            __builtin_amdgcn_sched_barrier(0);
+            float ds[16];
 #pragma unroll
-                        for (int bb = 0; bb < 4; ++bb) {
-                            const bool keep = static_cast<int>((w >> (8 * bb)) & 0xffu) >= p.thr8;
-                            dpt[4 * g + bb] = keep ? dpt[4 * g + bb] * p.zscale : 0.f;
-                        }
-                    }
-                }
+            for (int i = 0; i < 16; ++i) {
+                float pr;
+                if constexpr (MASK != kNoMask) pr = fast_exp2(fmaf(mk[i], kLog2e, st[i] * c) - lse);
+                else pr = fast_exp2(fmaf(st[i], c, -lse));
+                if (diag) pr = t0 + 32 * kb + c_row(i, h) <= qrow ? pr : 0.f;
+                ds[i] = pr;
+            }
+            if constexpr (DROPOUT) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) ds[i] *= dpt[i] - dlt;
+                for (int g = 0; g < 4; ++g) {
+                    const uint32_t w = dropout_word(p, bh, qrow, t0 + 32 * kb + 8 * g + 4 * h);
 #pragma unroll
-                for (int g = 0; g < 2; ++g) {
-                    const u32x4 bop = pack8<T>(&ds[8 * g]);
-#pragma unroll
-                    for (int db = 0; db < DB; ++db) {
-                        const u32x4 a = lds_read16(sKt, TransTile::read_off(32 * db + l32, 2 * kb + g, h));
-                        acc[db] = Mma<T>::run(a, bop, acc[db]);
+                    for (int bb = 0; bb < 4; ++bb) {
+                        const bool keep = static_cast<int>((w >> (8 * bb)) & 0xffu) >= p.thr8;
+                        dpt[4 * g + bb] = keep ? dpt[4 * g + bb] * p.zscale : 0.f;
                     }
                 }
             }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) ds[i] *= dpt[i] - dlt;
+            u32x4 bop[2];
+            bop[0] = pack8<T>(&ds[0]);
+            bop[1] = pack8<T>(&ds[8]);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 2 * DB; ++i) acc[i % DB] = Mma<T>::run(tf[i], bop[i / DB], acc[i % DB]);
         }
-        __syncthreads();
     }
 
     char* out = static_cast<char*>(p.dq) + (b * p.dqs[0] + hd * p.dqs[1] + static_cast<int64_t>(qrow) * p.dqs[2]) * 2;
@@ -576,12 +611,19 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv_pipe_kernel(const KParams p)
 }
 
 // ---------------------------------------------------------------------------------- launch
+template <typename T, int D, int NW, bool CAUSAL, int MASK>
+int launch_dq_waves(const KParams& p, hipStream_t stream) {
+    const dim3 grid(p.B * p.H * (p.S / (32 * NW))), block(64 * NW);
+    if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dq_kernel<T, D, NW, CAUSAL, MASK, true>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((mfma_dq_kernel<T, D, NW, CAUSAL, MASK, false>), grid, block, 0, stream, p);
+    return static_cast<int>(hipGetLastError());
+}
+
 template <typename T, int D, bool CAUSAL, int MASK>
 int launch_dq_dropout(const KParams& p, hipStream_t stream) {
-    const dim3 grid(p.B * p.H * (p.S / kBM)), block(256);
-    if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dq_kernel<T, D, CAUSAL, MASK, true>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((mfma_dq_kernel<T, D, CAUSAL, MASK, false>), grid, block, 0, stream, p);
-    return static_cast<int>(hipGetLastError());
+    // 8 waves (256 query rows) when the sequence allows it, else 4 waves (128 rows)
+    if (p.S % 256 == 0) return launch_dq_waves<T, D, 8, CAUSAL, MASK>(p, stream);
+    return launch_dq_waves<T, D, 4, CAUSAL, MASK>(p, stream);
 }
 
 template <typename T, int D, bool CAUSAL, int MASK>
