@@ -610,6 +610,212 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv_pipe_kernel(const KParams p)
         }
 }
 
+// ------------------------------------------------------------------ dK, dV (8 waves)
+// Same data flow as the dQ kernel with the roles of queries and keys exchanged: a workgroup of
+// NW waves owns 32*NW keys, one wave 32 of them with its K and V rows in registers (B operands)
+// and dK^T, dV^T in fp32 accumulators; two waves per SIMD. Q and dO stream as 64-row swizzled LDS
+// tiles (plus their lse and delta) in a ring of 4 filled by LDS-direct loads three tiles ahead.
+// Per 32-row query block: S = Q K^T and dP = dO V^T from row fragments, P and dS on the vector
+// ALU, dV^T += dO^T P and dK^T += Q^T dS with the transposed LDS reads of the same tiles.
+template <typename T, int D, int NW, bool CAUSAL, int MASK, bool DROPOUT>
+__global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParams p) {
+    using Tile = SwzTile<D>;
+    constexpr int kKeys = 32 * NW;
+    constexpr int kStages = 4;
+    constexpr int kStageBytes = 2 * Tile::kBytes + 2 * kBN * 4;  // Q tile, dO tile, lse, delta
+    constexpr int KK = D / 16;
+    constexpr int DB = D / 32;
+    constexpr int kBlocksPerWave = 2 * Tile::kBlocks / NW;
+    constexpr int kLoadsPerTile = kBlocksPerWave + 1;            // + lse or delta (upper bound per wave)
+    static_assert(2 * Tile::kBlocks % NW == 0, "tile blocks must divide among the waves");
+    __shared__ __attribute__((aligned(1024))) char smem[kStages * kStageBytes];
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+    int bh, kt;
+    map_block(blockIdx.x, p.B * p.H, p.S / kKeys, CAUSAL ? kHeavyFirst : kUniformTiles, &bh, &kt);
+    const int b = bh / p.H, hd = bh % p.H;
+    const int k0 = kt * kKeys;
+    const int wkey0 = k0 + 32 * wave;
+    const int key = wkey0 + l32;
+
+    const char* kbase = static_cast<const char*>(p.k) + (b * p.ks[0] + hd * p.ks[1]) * 2;
+    const char* vbase = static_cast<const char*>(p.v) + (b * p.vs[0] + hd * p.vs[1]) * 2;
+    const char* qbase = static_cast<const char*>(p.q) + (b * p.qs[0] + hd * p.qs[1]) * 2;
+    const char* gbase = static_cast<const char*>(p.d_o) + (b * p.dos[0] + hd * p.dos[1]) * 2;
+    const int64_t qrow_bytes = p.qs[2] * 2, grow_bytes = p.dos[2] * 2;
+    const float* lse_base = p.lse + static_cast<int64_t>(bh) * p.S;
+    const float* delta_base = p.delta + static_cast<int64_t>(bh) * p.S;
+
+    u32x4 kf[KK], vf[KK];
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+        kf[kk] = *reinterpret_cast<const u32x4*>(kbase + static_cast<int64_t>(key) * p.ks[2] * 2 + (2 * kk + h) * 16);
+        vf[kk] = *reinterpret_cast<const u32x4*>(vbase + static_cast<int64_t>(key) * p.vs[2] * 2 + (2 * kk + h) * 16);
+    }
+    const float c = p.scale_log2;
+
+    f32x16 dk[DB], dv[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+        dk[db] = zero16();
+        dv[db] = zero16();
+    }
+
+    int src_off[kBlocksPerWave];
+#pragma unroll
+    for (int i = 0; i < kBlocksPerWave; ++i) {
+        const int blk = wave * kBlocksPerWave + i;
+        const bool is_g = blk >= Tile::kBlocks;
+        src_off[i] = static_cast<int>(Tile::src_off(is_g ? blk - Tile::kBlocks : blk, lane, is_g ? grow_bytes : qrow_bytes));
+    }
+    const int t_begin = CAUSAL ? k0 / kBN : 0;                  // first tile with rows that see the workgroup's keys
+    const int my_begin = CAUSAL ? wkey0 / kBN : 0;              // first tile with rows that see this wave's keys
+    const int n_tiles = p.S / kBN;
+    auto issue_tile = [&](int t) {
+        char* stage = smem + (t % kStages) * kStageBytes;
+#pragma unroll
+        for (int i = 0; i < kBlocksPerWave; ++i) {
+            const int blk = wave * kBlocksPerWave + i;
+            const bool is_g = blk >= Tile::kBlocks;
+            const char* tile_src = is_g ? gbase + static_cast<int64_t>(t) * kBN * grow_bytes
+                                        : qbase + static_cast<int64_t>(t) * kBN * qrow_bytes;
+            char* dst = stage + (is_g ? Tile::kBytes + (blk - Tile::kBlocks) * 1024 : blk * 1024);
+            __builtin_amdgcn_global_load_lds(TRI_GLB_PTR(tile_src + src_off[i]), TRI_LDS_PTR(dst), 16, 0, 0);
+        }
+        if (wave == 0)
+            __builtin_amdgcn_global_load_lds(TRI_GLB_PTR(lse_base + t * kBN + lane), TRI_LDS_PTR(stage + 2 * Tile::kBytes), 4, 0, 0);
+        if (wave == NW - 1)
+            __builtin_amdgcn_global_load_lds(TRI_GLB_PTR(delta_base + t * kBN + lane),
+                                             TRI_LDS_PTR(stage + 2 * Tile::kBytes + kBN * 4), 4, 0, 0);
+    };
+    issue_tile(t_begin);
+    if (t_begin + 1 < n_tiles) issue_tile(t_begin + 1);
+    if (t_begin + 2 < n_tiles) issue_tile(t_begin + 2);
+
+    const int row_off0 = Tile::off(l32, h);
+    const int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
+
+    for (int j = t_begin; j < n_tiles; ++j) {
+        {
+            const int younger = min(2, n_tiles - 1 - j);
+            if (younger == 2) TRI_WAIT_VMCNT(2 * kLoadsPerTile);
+            else if (younger == 1) TRI_WAIT_VMCNT(kLoadsPerTile);
+            else TRI_WAIT_VMCNT(0);
+        }
+        __syncthreads();
+        if (j + 3 < n_tiles) issue_tile(j + 3);
+        if (j < my_begin) continue;
+
+        const char* sQ = smem + (j % kStages) * kStageBytes;
+        const char* sG = sQ + Tile::kBytes;
+        const float* sLse = reinterpret_cast<const float*>(sG + Tile::kBytes);
+        const float* sDelta = sLse + kBN;
+        const int r0 = j * kBN;
+        const bool diag = CAUSAL && r0 < wkey0 + 31;  // some row of the tile is above some key of the wave
+#pragma unroll 1
+        for (int qb = 0; qb < 2; ++qb) {
+            const int rb = r0 + 32 * qb;
+            if (CAUSAL && rb + 31 < wkey0) continue;  // whole block above the wave's keys
+            float mk[MASK != kNoMask ? 16 : 1];
+            if constexpr (MASK != kNoMask) {
+                const int64_t mbase = b * p.ms[0] + hd * p.ms[1] + key;
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    mk[i] = mask_at<T, MASK>(p.mask, mbase + static_cast<int64_t>(rb + c_row(i, h)) * p.ms[2]);
+            }
+            const int qoff = 32 * qb * Tile::kRowBytes;
+            u32x4 fr[KK];
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) fr[kk] = lds_read16(sQ, (row_off0 ^ (kk << 5)) + qoff);
+            __builtin_amdgcn_sched_barrier(0);
+            f32x16 s = zero16(), dp = zero16();
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) {
+                s = Mma<T>::run(fr[kk], kf[kk], s);
+                fr[kk] = lds_read16(sG, (row_off0 ^ (kk << 5)) + qoff);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) dp = Mma<T>::run(fr[kk], vf[kk], dp);
+            __builtin_amdgcn_sched_barrier(0);
+            u32x4 pb[2], sb[2];
+            {
+                float pr[16], ds[16];
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + 32 * qb + 8 * g + 4 * h);
+                    const f32x4 d4 = *reinterpret_cast<const f32x4*>(sDelta + 32 * qb + 8 * g + 4 * h);
+                    if constexpr (MASK != kNoMask) {
+#pragma unroll
+                        for (int bb = 0; bb < 4; ++bb) l4[bb] = l4[bb] == -INFINITY ? INFINITY : l4[bb];
+                    }
+                    uint32_t dw[4];
+                    if constexpr (DROPOUT) {
+                        const Philox4 r = dropout_block(p, bh, (rb + 8 * g + 4 * h) >> 2, key >> 2);
+#pragma unroll
+                        for (int bb = 0; bb < 4; ++bb) dw[bb] = (r.w[bb] >> (8 * (key & 3))) & 0xffu;
+                    }
+#pragma unroll
+                    for (int bb = 0; bb < 4; ++bb) {
+                        const int i = 4 * g + bb;
+                        float pv;
+                        if constexpr (MASK != kNoMask) pv = fast_exp2(fmaf(mk[i], kLog2e, s[i] * c) - l4[bb]);
+                        else pv = fast_exp2(fmaf(s[i], c, -l4[bb]));
+                        if (diag) pv = key <= rb + c_row(i, h) ? pv : 0.f;
+                        float dpv = dp[i];
+                        if constexpr (DROPOUT) {
+                            const bool keep = static_cast<int>(dw[bb]) >= p.thr8;
+                            dpv = keep ? dpv * p.zscale : 0.f;
+                            pr[i] = keep ? pv * p.zscale : 0.f;
+                        } else {
+                            pr[i] = pv;
+                        }
+                        ds[i] = pv * (dpv - d4[bb]);
+                    }
+                }
+#pragma unroll
+                for (int g = 0; g < 2; ++g) {
+                    pb[g] = pack8<T>(&pr[8 * g]);
+                    sb[g] = pack8<T>(&ds[8 * g]);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // dV^T += dO^T P, then dK^T += Q^T dS; DB transposed fragments in flight
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+                u32x4 tf[DB];
+#pragma unroll
+                for (int db = 0; db < DB; ++db) tf[db] = Tile::tr_frag(sG, tr_off0 ^ (db << 6), tr_off1 ^ (db << 6), 2 * qb + g);
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    dv[db] = Mma<T>::run(tf[db], pb[g], dv[db]);
+                    tf[db] = Tile::tr_frag(sQ, tr_off0 ^ (db << 6), tr_off1 ^ (db << 6), 2 * qb + g);
+                }
+#pragma unroll
+                for (int db = 0; db < DB; ++db) dk[db] = Mma<T>::run(tf[db], sb[g], dk[db]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+
+    char* dkrow = static_cast<char*>(p.dk) + (b * p.dks[0] + hd * p.dks[1] + static_cast<int64_t>(key) * p.dks[2]) * 2;
+    char* dvrow = static_cast<char*>(p.dv) + (b * p.dvs[0] + hd * p.dvs[1] + static_cast<int64_t>(key) * p.dvs[2]) * 2;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            u32x2 a, e;
+            a.x = Mma<T>::pack2(dk[db][4 * g + 0] * p.scale, dk[db][4 * g + 1] * p.scale);
+            a.y = Mma<T>::pack2(dk[db][4 * g + 2] * p.scale, dk[db][4 * g + 3] * p.scale);
+            e.x = Mma<T>::pack2(dv[db][4 * g + 0], dv[db][4 * g + 1]);
+            e.y = Mma<T>::pack2(dv[db][4 * g + 2], dv[db][4 * g + 3]);
+            *reinterpret_cast<u32x2*>(dkrow + (32 * db + 8 * g + 4 * h) * 2) = a;
+            *reinterpret_cast<u32x2*>(dvrow + (32 * db + 8 * g + 4 * h) * 2) = e;
+        }
+}
+
 // ---------------------------------------------------------------------------------- launch
 template <typename T, int D, int NW, bool CAUSAL, int MASK>
 int launch_dq_waves(const KParams& p, hipStream_t stream) {
@@ -626,15 +832,31 @@ int launch_dq_dropout(const KParams& p, hipStream_t stream) {
     return launch_dq_waves<T, D, 4, CAUSAL, MASK>(p, stream);
 }
 
+template <typename T, int D, int NW, bool CAUSAL, int MASK>
+int launch_dkdv_waves(const KParams& p, hipStream_t stream) {
+    const dim3 grid(p.B * p.H * (p.S / (32 * NW))), block(64 * NW);
+    if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dkdv_wide_kernel<T, D, NW, CAUSAL, MASK, true>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((mfma_dkdv_wide_kernel<T, D, NW, CAUSAL, MASK, false>), grid, block, 0, stream, p);
+    return static_cast<int>(hipGetLastError());
+}
+
 template <typename T, int D, bool CAUSAL, int MASK>
 int launch_dkdv_dropout(const KParams& p, hipStream_t stream) {
-    const dim3 grid(p.B * p.H * (p.S / kBM)), block(256);
-    // The software-pipelined kernel is used where it is the faster one (no mask, no dropout: those
-    // variants need more registers than its one-wave-per-SIMD schedule leaves free).
-    if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, CAUSAL, MASK, true>), grid, block, 0, stream, p);
-    else if (MASK != kNoMask) hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, CAUSAL, MASK, false>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((mfma_dkdv_pipe_kernel<T, D, CAUSAL, kNoMask, false>), grid, block, 0, stream, p);
-    return static_cast<int>(hipGetLastError());
+    if constexpr (D == 64) {
+        // the two-waves-per-SIMD kernel fits its registers: 8 waves (256 keys) when the sequence
+        // allows it, else 4 waves (128 keys)
+        if (p.S % 256 == 0) return launch_dkdv_waves<T, D, 8, CAUSAL, MASK>(p, stream);
+        return launch_dkdv_waves<T, D, 4, CAUSAL, MASK>(p, stream);
+    } else {
+        // D = 128: K, V and both gradient accumulators of a 32-key block take 192 registers, too many
+        // for two waves per SIMD; the one-wave pipelined kernel serves the plain and causal variants,
+        // the mask and dropout variants (which need still more registers) keep the staged kernel
+        const dim3 grid(p.B * p.H * (p.S / kBM)), block(256);
+        if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, CAUSAL, MASK, true>), grid, block, 0, stream, p);
+        else if (MASK != kNoMask) hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, CAUSAL, MASK, false>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((mfma_dkdv_pipe_kernel<T, D, CAUSAL, kNoMask, false>), grid, block, 0, stream, p);
+        return static_cast<int>(hipGetLastError());
+    }
 }
 
 template <int WHICH, typename T, int D, bool CAUSAL, int MASK>
