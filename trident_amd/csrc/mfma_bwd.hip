@@ -816,6 +816,241 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
         }
 }
 
+// ------------------------------------------------------------------ dK, dV (paired waves)
+// For D = 128 the K and V rows plus both gradient accumulators of a 32-key block need 192
+// registers, which rules out two waves per SIMD. Here two waves share a key block instead: a
+// workgroup of 8 waves owns 128 keys; waves w and w+4 both hold the K and V rows of key block w%4.
+// Per 64-row tile of Q and dO (swizzled LDS ring filled by LDS-direct loads, as in the dQ kernel)
+//   phase 1: member m of a pair computes S, dP, P and dS of query block m (16 MFMA + softmax)
+//            and leaves P and dS, already packed as B operands, in an LDS exchange slot;
+//   phase 2: after a barrier each member accumulates, for BOTH query blocks, the half of the head
+//            dimension it owns: dV^T[2m..2m+1] += dO^T P, dK^T[2m..2m+1] += Q^T dS (16 MFMA).
+// No MFMA is executed twice, and a wave keeps only 128 persistent registers.
+template <typename T, int D, bool CAUSAL, int MASK, bool DROPOUT>
+__global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p) {
+    using Tile = SwzTile<D>;
+    constexpr int NW = 8;
+    constexpr int kKeys = 128;
+    constexpr int kStages = 3;
+    constexpr int kStageBytes = 2 * Tile::kBytes + 2 * kBN * 4;  // Q tile, dO tile, lse, delta
+    constexpr int kXchBytes = NW * 4 * 1024;                     // per wave: P[2], dS[2] fragments
+    constexpr int KK = D / 16;
+    constexpr int DB = D / 32;
+    constexpr int DH = DB / 2;                                   // column blocks a pair member accumulates
+    constexpr int kBlocksPerWave = 2 * Tile::kBlocks / NW;
+    constexpr int kLoadsPerTile = kBlocksPerWave + 1;
+    __shared__ __attribute__((aligned(1024))) char smem[kStages * kStageBytes + kXchBytes];
+    char* xch = smem + kStages * kStageBytes;
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int kb = wave & 3, member = wave >> 2;
+    const int lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+    int bh, kt;
+    map_block(blockIdx.x, p.B * p.H, p.S / kKeys, CAUSAL ? kHeavyFirst : kUniformTiles, &bh, &kt);
+    const int b = bh / p.H, hd = bh % p.H;
+    const int k0 = kt * kKeys;
+    const int wkey0 = k0 + 32 * kb;
+    const int key = wkey0 + l32;
+
+    const char* kbase = static_cast<const char*>(p.k) + (b * p.ks[0] + hd * p.ks[1]) * 2;
+    const char* vbase = static_cast<const char*>(p.v) + (b * p.vs[0] + hd * p.vs[1]) * 2;
+    const char* qbase = static_cast<const char*>(p.q) + (b * p.qs[0] + hd * p.qs[1]) * 2;
+    const char* gbase = static_cast<const char*>(p.d_o) + (b * p.dos[0] + hd * p.dos[1]) * 2;
+    const int64_t qrow_bytes = p.qs[2] * 2, grow_bytes = p.dos[2] * 2;
+    const float* lse_base = p.lse + static_cast<int64_t>(bh) * p.S;
+    const float* delta_base = p.delta + static_cast<int64_t>(bh) * p.S;
+
+    u32x4 kf[KK], vf[KK];
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+        kf[kk] = *reinterpret_cast<const u32x4*>(kbase + static_cast<int64_t>(key) * p.ks[2] * 2 + (2 * kk + h) * 16);
+        vf[kk] = *reinterpret_cast<const u32x4*>(vbase + static_cast<int64_t>(key) * p.vs[2] * 2 + (2 * kk + h) * 16);
+    }
+    const float c = p.scale_log2;
+
+    f32x16 dk[DH], dv[DH];
+#pragma unroll
+    for (int d = 0; d < DH; ++d) {
+        dk[d] = zero16();
+        dv[d] = zero16();
+    }
+
+    int src_off[kBlocksPerWave];
+#pragma unroll
+    for (int i = 0; i < kBlocksPerWave; ++i) {
+        const int blk = wave * kBlocksPerWave + i;
+        const bool is_g = blk >= Tile::kBlocks;
+        src_off[i] = static_cast<int>(Tile::src_off(is_g ? blk - Tile::kBlocks : blk, lane, is_g ? grow_bytes : qrow_bytes));
+    }
+    const int t_begin = CAUSAL ? k0 / kBN : 0;
+    const int n_tiles = p.S / kBN;
+    auto issue_tile = [&](int t) {
+        char* stage = smem + (t % kStages) * kStageBytes;
+#pragma unroll
+        for (int i = 0; i < kBlocksPerWave; ++i) {
+            const int blk = wave * kBlocksPerWave + i;
+            const bool is_g = blk >= Tile::kBlocks;
+            const char* tile_src = is_g ? gbase + static_cast<int64_t>(t) * kBN * grow_bytes
+                                        : qbase + static_cast<int64_t>(t) * kBN * qrow_bytes;
+            char* dst = stage + (is_g ? Tile::kBytes + (blk - Tile::kBlocks) * 1024 : blk * 1024);
+            __builtin_amdgcn_global_load_lds(TRI_GLB_PTR(tile_src + src_off[i]), TRI_LDS_PTR(dst), 16, 0, 0);
+        }
+        if (wave == 0)
+            __builtin_amdgcn_global_load_lds(TRI_GLB_PTR(lse_base + t * kBN + lane), TRI_LDS_PTR(stage + 2 * Tile::kBytes), 4, 0, 0);
+        if (wave == NW - 1)
+            __builtin_amdgcn_global_load_lds(TRI_GLB_PTR(delta_base + t * kBN + lane),
+                                             TRI_LDS_PTR(stage + 2 * Tile::kBytes + kBN * 4), 4, 0, 0);
+    };
+    issue_tile(t_begin);
+    if (t_begin + 1 < n_tiles) issue_tile(t_begin + 1);
+
+    const int row_off0 = Tile::off(l32, h);
+    const int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
+    char* my_xch = xch + wave * 4096 + lane * 16;
+    const char* peer_xch = xch + (wave ^ 4) * 4096 + lane * 16;
+
+    for (int j = t_begin; j < n_tiles; ++j) {
+        // tile j has landed (tile j+1 may still be in flight) and is visible; every wave is done with
+        // tile j-1 and with the exchange slots, so tile j+2 may overwrite the slot of tile j-1
+        if (j + 1 < n_tiles) TRI_WAIT_VMCNT(kLoadsPerTile);
+        else TRI_WAIT_VMCNT(0);
+        __syncthreads();
+        if (j + 2 < n_tiles) issue_tile(j + 2);
+
+        const char* sQ = smem + (j % kStages) * kStageBytes;
+        const char* sG = sQ + Tile::kBytes;
+        const float* sLse = reinterpret_cast<const float*>(sG + Tile::kBytes);
+        const float* sDelta = sLse + kBN;
+        const int r0 = j * kBN;
+        const int rb = r0 + 32 * member;  // first row of the query block this wave scores
+
+        // ---- phase 1: P and dS of query block `member` against this pair's keys
+        u32x4 pb[2], sb[2];
+        if (!CAUSAL || rb + 31 >= wkey0) {
+            const bool diag = CAUSAL && rb < wkey0 + 31;
+            float mk[MASK != kNoMask ? 16 : 1];
+            if constexpr (MASK != kNoMask) {
+                const int64_t mbase = b * p.ms[0] + hd * p.ms[1] + key;
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    mk[i] = mask_at<T, MASK>(p.mask, mbase + static_cast<int64_t>(rb + c_row(i, h)) * p.ms[2]);
+            }
+            const int qoff = 32 * member * Tile::kRowBytes;
+            u32x4 fr[KK];
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) fr[kk] = lds_read16(sQ, (row_off0 ^ (kk << 5)) + qoff);
+            __builtin_amdgcn_sched_barrier(0);
+            f32x16 s = zero16(), dp = zero16();
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) {
+                s = Mma<T>::run(fr[kk], kf[kk], s);
+                fr[kk] = lds_read16(sG, (row_off0 ^ (kk << 5)) + qoff);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) dp = Mma<T>::run(fr[kk], vf[kk], dp);
+            __builtin_amdgcn_sched_barrier(0);
+            float pr[16], ds[16];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + 32 * member + 8 * g + 4 * h);
+                const f32x4 d4 = *reinterpret_cast<const f32x4*>(sDelta + 32 * member + 8 * g + 4 * h);
+                if constexpr (MASK != kNoMask) {
+#pragma unroll
+                    for (int bb = 0; bb < 4; ++bb) l4[bb] = l4[bb] == -INFINITY ? INFINITY : l4[bb];
+                }
+                uint32_t dw[4];
+                if constexpr (DROPOUT) {
+                    const Philox4 r = dropout_block(p, bh, (rb + 8 * g + 4 * h) >> 2, key >> 2);
+#pragma unroll
+                    for (int bb = 0; bb < 4; ++bb) dw[bb] = (r.w[bb] >> (8 * (key & 3))) & 0xffu;
+                }
+#pragma unroll
+                for (int bb = 0; bb < 4; ++bb) {
+                    const int i = 4 * g + bb;
+                    float pv;
+                    if constexpr (MASK != kNoMask) pv = fast_exp2(fmaf(mk[i], kLog2e, s[i] * c) - l4[bb]);
+                    else pv = fast_exp2(fmaf(s[i], c, -l4[bb]));
+                    if (diag) pv = key <= rb + c_row(i, h) ? pv : 0.f;
+                    float dpv = dp[i];
+                    if constexpr (DROPOUT) {
+                        const bool keep = static_cast<int>(dw[bb]) >= p.thr8;
+                        dpv = keep ? dpv * p.zscale : 0.f;
+                        pr[i] = keep ? pv * p.zscale : 0.f;
+                    } else {
+                        pr[i] = pv;
+                    }
+                    ds[i] = pv * (dpv - d4[bb]);
+                }
+            }
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+                pb[g] = pack8<T>(&pr[8 * g]);
+                sb[g] = pack8<T>(&ds[8 * g]);
+            }
+        } else {
+#pragma unroll
+            for (int g = 0; g < 2; ++g) pb[g] = sb[g] = u32x4{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            *reinterpret_cast<u32x4*>(my_xch + g * 1024) = pb[g];
+            *reinterpret_cast<u32x4*>(my_xch + (2 + g) * 1024) = sb[g];
+        }
+        __syncthreads();
+
+        // ---- phase 2: this member's half of the head dimension, both query blocks
+        if (!CAUSAL || r0 + kBN - 1 >= wkey0) {
+            u32x4 pp[2], ps[2];  // the partner's P and dS
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+                pp[g] = *reinterpret_cast<const u32x4*>(peer_xch + g * 1024);
+                ps[g] = *reinterpret_cast<const u32x4*>(peer_xch + (2 + g) * 1024);
+            }
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb) {
+#pragma unroll
+                for (int g = 0; g < 2; ++g) {
+                    const u32x4 bp = qb == member ? pb[g] : pp[g];
+                    const u32x4 bs = qb == member ? sb[g] : ps[g];
+                    u32x4 tf[DH];
+#pragma unroll
+                    for (int d = 0; d < DH; ++d) {
+                        const int db = DH * member + d;
+                        tf[d] = Tile::tr_frag(sG, tr_off0 ^ (db << 6), tr_off1 ^ (db << 6), 2 * qb + g);
+                    }
+#pragma unroll
+                    for (int d = 0; d < DH; ++d) {
+                        const int db = DH * member + d;
+                        dv[d] = Mma<T>::run(tf[d], bp, dv[d]);
+                        tf[d] = Tile::tr_frag(sQ, tr_off0 ^ (db << 6), tr_off1 ^ (db << 6), 2 * qb + g);
+                    }
+#pragma unroll
+                    for (int d = 0; d < DH; ++d) dk[d] = Mma<T>::run(tf[d], bs, dk[d]);
+                }
+            }
+        }
+    }
+
+    char* dkrow = static_cast<char*>(p.dk) + (b * p.dks[0] + hd * p.dks[1] + static_cast<int64_t>(key) * p.dks[2]) * 2;
+    char* dvrow = static_cast<char*>(p.dv) + (b * p.dvs[0] + hd * p.dvs[1] + static_cast<int64_t>(key) * p.dvs[2]) * 2;
+#pragma unroll
+    for (int d = 0; d < DH; ++d) {
+        const int db = DH * member + d;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            u32x2 a, e;
+            a.x = Mma<T>::pack2(dk[d][4 * g + 0] * p.scale, dk[d][4 * g + 1] * p.scale);
+            a.y = Mma<T>::pack2(dk[d][4 * g + 2] * p.scale, dk[d][4 * g + 3] * p.scale);
+            e.x = Mma<T>::pack2(dv[d][4 * g + 0], dv[d][4 * g + 1]);
+            e.y = Mma<T>::pack2(dv[d][4 * g + 2], dv[d][4 * g + 3]);
+            *reinterpret_cast<u32x2*>(dkrow + (32 * db + 8 * g + 4 * h) * 2) = a;
+            *reinterpret_cast<u32x2*>(dvrow + (32 * db + 8 * g + 4 * h) * 2) = e;
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------------- launch
 template <typename T, int D, int NW, bool CAUSAL, int MASK>
 int launch_dq_waves(const KParams& p, hipStream_t stream) {
@@ -854,7 +1089,7 @@ int launch_dkdv_dropout(const KParams& p, hipStream_t stream) {
         const dim3 grid(p.B * p.H * (p.S / kBM)), block(256);
         if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, CAUSAL, MASK, true>), grid, block, 0, stream, p);
         else if (MASK != kNoMask) hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, CAUSAL, MASK, false>), grid, block, 0, stream, p);
-        else hipLaunchKernelGGL((mfma_dkdv_pipe_kernel<T, D, CAUSAL, kNoMask, false>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((mfma_dkdv_pair_kernel<T, D, CAUSAL, kNoMask, false>), grid, dim3(512), 0, stream, p);
         return static_cast<int>(hipGetLastError());
     }
 }
