@@ -72,6 +72,13 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
     if (lse == -INFINITY) lse = INFINITY;  // fully masked row: every probability is 0
     const float dlt = p.delta[static_cast<int64_t>(bh) * p.S + qrow];
     const float c = p.scale_log2;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+        settle(qf[kk]);
+        settle(gf[kk]);
+    }
+    settle(lse);
+    settle(dlt);
 
     f32x16 acc[DB];
 #pragma unroll
@@ -95,7 +102,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
             const bool is_v = blk >= Tile::kBlocks;
             const char* tile_src = is_v ? vbase + static_cast<int64_t>(t) * kBN * vrow_bytes
                                         : kbase + static_cast<int64_t>(t) * kBN * krow_bytes;
-            __builtin_amdgcn_global_load_lds(TRI_GLB_PTR(tile_src + src_off[i]), TRI_LDS_PTR(stage + blk * 1024), 16, 0, 0);
+            lds_direct_load16(tile_src + src_off[i], stage + blk * 1024);
         }
     };
     issue_tile(0);
@@ -114,7 +121,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
             else if (younger == 1) TRI_WAIT_VMCNT(kBlocksPerWave);
             else TRI_WAIT_VMCNT(0);
         }
-        __syncthreads();
+        lds_barrier();
         if (j + 3 < n_tiles) issue_tile(j + 3);
         if (j >= my_tiles) continue;
 
@@ -350,266 +357,6 @@ __global__ __launch_bounds__(256, 2) void mfma_dkdv_kernel(const KParams p) {
         }
 }
 
-// ------------------------------------------------------------------- dK, dV (pipelined)
-// One wave per SIMD with the full register file: a workgroup of 4 waves owns 128 keys, a wave
-// 32 of them with its K and V rows in registers (B operands) and dK^T, dV^T in fp32
-// accumulators. Q and dO stream as 64-row swizzled LDS tiles filled by LDS-direct loads two
-// tiles ahead (ring of 4). Per 32-row query block a wave issues
-//   stage 1: S = Q K^T and dP = dO V^T                     (16 MFMA, row fragments)
-//   stage 2: P = exp2(S c - lse), dS = P (dP - delta)       (vector ALU)
-//   stage 3: dV^T += dO^T P and dK^T += Q^T dS              (16 MFMA, transposed fragments)
-// and the loop is software-pipelined inside the wave: stage 3 of the previous block is
-// interleaved, MFMA by MFMA, with stage 2 of the current one, and every LDS fragment is
-// requested eight MFMAs before it is used, so neither the vector ALU nor the LDS latency
-// leaves the matrix pipe idle.
-template <typename T, int D, bool CAUSAL, int MASK, bool DROPOUT>
-__global__ __launch_bounds__(256, 1) void mfma_dkdv_pipe_kernel(const KParams p) {
-    using Tile = SwzTile<D>;
-    constexpr int kKeys = 128;
-    constexpr int kStages = 4;
-    constexpr int kStageBytes = 2 * Tile::kBytes + 2 * kBN * 4;  // Q tile, dO tile, lse, delta
-    constexpr int KK = D / 16;
-    constexpr int DB = D / 32;
-    constexpr int kBlocksPerWave = 2 * Tile::kBlocks / 4;        // LDS-direct loads per wave and tile
-    constexpr int kLoadsPerTile = kBlocksPerWave + 1;            // + lse or delta (upper bound per wave)
-    constexpr int NF = 2 * DB;                                   // transposed fragments per operand and block
-    __shared__ __attribute__((aligned(1024))) char smem[kStages * kStageBytes];
-
-    const int tid = threadIdx.x;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int lane = tid & 63, l32 = lane & 31, h = lane >> 5;
-    int bh, kt;
-    map_block(blockIdx.x, p.B * p.H, p.S / kKeys, CAUSAL ? kHeavyFirst : kUniformTiles, &bh, &kt);
-    const int b = bh / p.H, hd = bh % p.H;
-    const int k0 = kt * kKeys;
-    const int wkey0 = k0 + 32 * wave;
-    const int key = wkey0 + l32;
-
-    const char* kbase = static_cast<const char*>(p.k) + (b * p.ks[0] + hd * p.ks[1]) * 2;
-    const char* vbase = static_cast<const char*>(p.v) + (b * p.vs[0] + hd * p.vs[1]) * 2;
-    const char* qbase = static_cast<const char*>(p.q) + (b * p.qs[0] + hd * p.qs[1]) * 2;
-    const char* gbase = static_cast<const char*>(p.d_o) + (b * p.dos[0] + hd * p.dos[1]) * 2;
-    const int64_t qrow_bytes = p.qs[2] * 2, grow_bytes = p.dos[2] * 2;
-    const float* lse_base = p.lse + static_cast<int64_t>(bh) * p.S;
-    const float* delta_base = p.delta + static_cast<int64_t>(bh) * p.S;
-
-    u32x4 kf[KK], vf[KK];
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-        kf[kk] = *reinterpret_cast<const u32x4*>(kbase + static_cast<int64_t>(key) * p.ks[2] * 2 + (2 * kk + h) * 16);
-        vf[kk] = *reinterpret_cast<const u32x4*>(vbase + static_cast<int64_t>(key) * p.vs[2] * 2 + (2 * kk + h) * 16);
-    }
-    const float c = p.scale_log2;
-
-    f32x16 dk[DB], dv[DB];
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-        dk[db] = zero16();
-        dv[db] = zero16();
-    }
-
-    int src_off[kBlocksPerWave];
-#pragma unroll
-    for (int i = 0; i < kBlocksPerWave; ++i) {
-        const int blk = wave * kBlocksPerWave + i;
-        const bool is_g = blk >= Tile::kBlocks;
-        src_off[i] = static_cast<int>(Tile::src_off(is_g ? blk - Tile::kBlocks : blk, lane, is_g ? grow_bytes : qrow_bytes));
-    }
-    const int t_begin = CAUSAL ? k0 / kBN : 0;  // first 64-row tile with visible rows
-    const int n_tiles = p.S / kBN;
-    auto issue_tile = [&](int t) {
-        char* stage = smem + (t % kStages) * kStageBytes;
-#pragma unroll
-        for (int i = 0; i < kBlocksPerWave; ++i) {
-            const int blk = wave * kBlocksPerWave + i;
-            const bool is_g = blk >= Tile::kBlocks;
-            const char* tile_src = is_g ? gbase + static_cast<int64_t>(t) * kBN * grow_bytes
-                                        : qbase + static_cast<int64_t>(t) * kBN * qrow_bytes;
-            char* dst = stage + (is_g ? Tile::kBytes + (blk - Tile::kBlocks) * 1024 : blk * 1024);
-            __builtin_amdgcn_global_load_lds(TRI_GLB_PTR(tile_src + src_off[i]), TRI_LDS_PTR(dst), 16, 0, 0);
-        }
-        if (wave == 0)
-            __builtin_amdgcn_global_load_lds(TRI_GLB_PTR(lse_base + t * kBN + lane), TRI_LDS_PTR(stage + 2 * Tile::kBytes), 4, 0, 0);
-        if (wave == 3)
-            __builtin_amdgcn_global_load_lds(TRI_GLB_PTR(delta_base + t * kBN + lane),
-                                             TRI_LDS_PTR(stage + 2 * Tile::kBytes + kBN * 4), 4, 0, 0);
-    };
-    // tiles t_begin .. t_begin+2 in flight; tile t_begin (and the K/V fragments) landed
-    issue_tile(t_begin);
-    if (t_begin + 1 < n_tiles) issue_tile(t_begin + 1);
-    if (t_begin + 2 < n_tiles) issue_tile(t_begin + 2);
-    {
-        const int later = min(2, n_tiles - 1 - t_begin);
-        if (later == 2) TRI_WAIT_VMCNT(2 * kLoadsPerTile);
-        else if (later == 1) TRI_WAIT_VMCNT(kLoadsPerTile);
-        else TRI_WAIT_VMCNT(0);
-    }
-    __syncthreads();
-
-    const int row_off0 = Tile::off(l32, h);
-    const int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
-    auto q_tile = [&](int u) { return smem + ((u >> 1) % kStages) * kStageBytes; };
-    // row fragment kk of query block u (is_g: dO instead of Q)
-    auto row_frag = [&](int u, bool is_g, int kk) {
-        return lds_read16(q_tile(u) + (is_g ? Tile::kBytes : 0), (row_off0 ^ (kk << 5)) + 32 * (u & 1) * Tile::kRowBytes);
-    };
-    // transposed fragment f = 2*db... of query block u: index i in [0,NF): K-step g = i / DB, column block db = i % DB
-    auto tr_frag = [&](int u, bool is_g, int i) {
-        const int db = i % DB, g = i / DB;
-        return Tile::tr_frag(q_tile(u) + (is_g ? Tile::kBytes : 0), tr_off0 ^ (db << 6), tr_off1 ^ (db << 6), 2 * (u & 1) + g);
-    };
-
-    const int u_begin = 2 * t_begin, u_end = 2 * n_tiles;
-    const int u_diag = wkey0 >> 5;  // query blocks up to this one need the element-wise causal test
-
-    u32x4 ring[KK];   // row fragments, requested one operand ahead
-    u32x4 tring[NF];  // transposed fragments, requested one operand ahead
-    f32x16 sacc, dpacc;
-    u32x4 pb[2][2], sb[2][2];  // [parity of the block][K-step]: P and dS as B operands
-
-    // stage 1 of block u: ring holds Q fragments of u on entry and Q fragments of u+1 on exit
-    auto stage1 = [&](int u) {
-        sacc = zero16();
-        dpacc = zero16();
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-            sacc = Mma<T>::run(ring[kk], kf[kk], sacc);
-            ring[kk] = row_frag(u, true, kk);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-            dpacc = Mma<T>::run(ring[kk], vf[kk], dpacc);
-            if (u + 1 < u_end) ring[kk] = row_frag(u + 1, false, kk);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    };
-    // stage 2 for elements [4g, 4g+4) of block u (one group of four consecutive query rows)
-    float pr[16], ds[16];
-    float mk[MASK != kNoMask ? 16 : 1];
-    auto load_mask = [&](int u) {
-        if constexpr (MASK != kNoMask) {
-            const int64_t mbase = b * p.ms[0] + hd * p.ms[1] + key;
-#pragma unroll
-            for (int i = 0; i < 16; ++i)
-                mk[i] = mask_at<T, MASK>(p.mask, mbase + static_cast<int64_t>(32 * u + c_row(i, h)) * p.ms[2]);
-        }
-    };
-    auto stage2_group = [&](int u, int g) {
-        const float* sLse = reinterpret_cast<const float*>(q_tile(u) + 2 * Tile::kBytes);
-        const float* sDelta = sLse + kBN;
-        f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + 32 * (u & 1) + 8 * g + 4 * h);
-        const f32x4 d4 = *reinterpret_cast<const f32x4*>(sDelta + 32 * (u & 1) + 8 * g + 4 * h);
-        if constexpr (MASK != kNoMask) {
-#pragma unroll
-            for (int bb = 0; bb < 4; ++bb) l4[bb] = l4[bb] == -INFINITY ? INFINITY : l4[bb];
-        }
-        uint32_t dw[4];
-        if constexpr (DROPOUT) {
-            const Philox4 r = dropout_block(p, bh, (32 * u + 8 * g + 4 * h) >> 2, key >> 2);
-#pragma unroll
-            for (int bb = 0; bb < 4; ++bb) dw[bb] = (r.w[bb] >> (8 * (key & 3))) & 0xffu;
-        }
-        const bool diag = CAUSAL && u <= u_diag;
-#pragma unroll
-        for (int bb = 0; bb < 4; ++bb) {
-            const int i = 4 * g + bb;
-            float pv;
-            if constexpr (MASK != kNoMask) pv = fast_exp2(fmaf(mk[i], kLog2e, sacc[i] * c) - l4[bb]);
-            else pv = fast_exp2(fmaf(sacc[i], c, -l4[bb]));
-            if (diag) pv = key <= 32 * u + c_row(i, h) ? pv : 0.f;
-            float dpv = dpacc[i];
-            if constexpr (DROPOUT) {
-                const bool keep = static_cast<int>(dw[bb]) >= p.thr8;
-                dpv = keep ? dpv * p.zscale : 0.f;
-                pr[i] = keep ? pv * p.zscale : 0.f;
-            } else {
-                pr[i] = pv;
-            }
-            ds[i] = pv * (dpv - d4[bb]);
-        }
-    };
-    auto pack_block = [&](int par) {
-#pragma unroll
-        for (int g = 0; g < 2; ++g) {
-            pb[par][g] = pack8<T>(&pr[8 * g]);
-            sb[par][g] = pack8<T>(&ds[8 * g]);
-        }
-    };
-    // stage 3 of block u (parity par); tring holds dO^T fragments of u on entry and of u+1 on exit.
-    // `with_stage2`: interleave stage 2 of block u+1 between the MFMAs.
-    auto stage3 = [&](int u, int par, bool with_stage2) {
-#pragma unroll
-        for (int i = 0; i < NF; ++i) {
-            dv[i % DB] = Mma<T>::run(tring[i], pb[par][i / DB], dv[i % DB]);
-            tring[i] = tr_frag(u, false, i);
-            if (with_stage2 && (i % (NF / 2)) == 0) stage2_group(u + 1, i / (NF / 2));
-            __builtin_amdgcn_sched_barrier(0);
-        }
-#pragma unroll
-        for (int i = 0; i < NF; ++i) {
-            dk[i % DB] = Mma<T>::run(tring[i], sb[par][i / DB], dk[i % DB]);
-            if (u + 1 < u_end) tring[i] = tr_frag(u + 1, true, i);
-            if (with_stage2 && (i % (NF / 2)) == 0) stage2_group(u + 1, 2 + i / (NF / 2));
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    };
-
-    // ---- prologue: first block without overlap
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) ring[kk] = row_frag(u_begin, false, kk);
-#pragma unroll
-    for (int i = 0; i < NF; ++i) tring[i] = tr_frag(u_begin, true, i);
-    load_mask(u_begin);
-    stage1(u_begin);
-#pragma unroll
-    for (int g = 0; g < 4; ++g) stage2_group(u_begin, g);
-    pack_block(0);
-
-    // ---- steady state: block u's stage 1, then stage 3 of u-1 interleaved with stage 2 of u.
-    // Two blocks (one tile) per trip so that the P/dS buffers alternate statically.
-    for (int u = u_begin + 1; u < u_end; u += 2) {
-        {
-            // u is odd: block u+1 starts tile (u+1)/2, which must have landed and be visible to all
-            // waves; the slot of tile (u-3)/2 is free again and takes the load of tile (u+5)/2
-            const int t_new = (u + 1) >> 1;
-            if (t_new < n_tiles) {
-                if (t_new + 1 < n_tiles) TRI_WAIT_VMCNT(kLoadsPerTile);
-                else TRI_WAIT_VMCNT(0);
-                __syncthreads();
-                if (t_new + 2 < n_tiles) issue_tile(t_new + 2);
-            }
-        }
-        load_mask(u);
-        stage1(u);
-        stage3(u - 1, 0, true);
-        pack_block(1);
-        if (u + 1 < u_end) {
-            load_mask(u + 1);
-            stage1(u + 1);
-            stage3(u, 1, true);
-            pack_block(0);
-        }
-    }
-    // ---- drain: the last block is odd
-    stage3(u_end - 1, 1, false);
-
-    char* dkrow = static_cast<char*>(p.dk) + (b * p.dks[0] + hd * p.dks[1] + static_cast<int64_t>(key) * p.dks[2]) * 2;
-    char* dvrow = static_cast<char*>(p.dv) + (b * p.dvs[0] + hd * p.dvs[1] + static_cast<int64_t>(key) * p.dvs[2]) * 2;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            u32x2 a, e;
-            a.x = Mma<T>::pack2(dk[db][4 * g + 0] * p.scale, dk[db][4 * g + 1] * p.scale);
-            a.y = Mma<T>::pack2(dk[db][4 * g + 2] * p.scale, dk[db][4 * g + 3] * p.scale);
-            e.x = Mma<T>::pack2(dv[db][4 * g + 0], dv[db][4 * g + 1]);
-            e.y = Mma<T>::pack2(dv[db][4 * g + 2], dv[db][4 * g + 3]);
-            *reinterpret_cast<u32x2*>(dkrow + (32 * db + 8 * g + 4 * h) * 2) = a;
-            *reinterpret_cast<u32x2*>(dvrow + (32 * db + 8 * g + 4 * h) * 2) = e;
-        }
-}
-
 // ------------------------------------------------------------------ dK, dV (8 waves)
 // Same data flow as the dQ kernel with the roles of queries and keys exchanged: a workgroup of
 // NW waves owns 32*NW keys, one wave 32 of them with its K and V rows in registers (B operands)
@@ -654,6 +401,11 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
         kf[kk] = *reinterpret_cast<const u32x4*>(kbase + static_cast<int64_t>(key) * p.ks[2] * 2 + (2 * kk + h) * 16);
         vf[kk] = *reinterpret_cast<const u32x4*>(vbase + static_cast<int64_t>(key) * p.vs[2] * 2 + (2 * kk + h) * 16);
     }
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+        settle(kf[kk]);
+        settle(vf[kk]);
+    }
     const float c = p.scale_log2;
 
     f32x16 dk[DB], dv[DB];
@@ -682,13 +434,12 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
             const char* tile_src = is_g ? gbase + static_cast<int64_t>(t) * kBN * grow_bytes
                                         : qbase + static_cast<int64_t>(t) * kBN * qrow_bytes;
             char* dst = stage + (is_g ? Tile::kBytes + (blk - Tile::kBlocks) * 1024 : blk * 1024);
-            __builtin_amdgcn_global_load_lds(TRI_GLB_PTR(tile_src + src_off[i]), TRI_LDS_PTR(dst), 16, 0, 0);
+            lds_direct_load16(tile_src + src_off[i], dst);
         }
         if (wave == 0)
-            __builtin_amdgcn_global_load_lds(TRI_GLB_PTR(lse_base + t * kBN + lane), TRI_LDS_PTR(stage + 2 * Tile::kBytes), 4, 0, 0);
+            lds_direct_load4(lse_base + t * kBN + lane, stage + 2 * Tile::kBytes);
         if (wave == NW - 1)
-            __builtin_amdgcn_global_load_lds(TRI_GLB_PTR(delta_base + t * kBN + lane),
-                                             TRI_LDS_PTR(stage + 2 * Tile::kBytes + kBN * 4), 4, 0, 0);
+            lds_direct_load4(delta_base + t * kBN + lane, stage + 2 * Tile::kBytes + kBN * 4);
     };
     issue_tile(t_begin);
     if (t_begin + 1 < n_tiles) issue_tile(t_begin + 1);
@@ -704,7 +455,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
             else if (younger == 1) TRI_WAIT_VMCNT(kLoadsPerTile);
             else TRI_WAIT_VMCNT(0);
         }
-        __syncthreads();
+        lds_barrier();
         if (j + 3 < n_tiles) issue_tile(j + 3);
         if (j < my_begin) continue;
 
@@ -821,10 +572,10 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
 // registers, which rules out two waves per SIMD. Here two waves share a key block instead: a
 // workgroup of 8 waves owns 128 keys; waves w and w+4 both hold the K and V rows of key block w%4.
 // Per 64-row tile of Q and dO (swizzled LDS ring filled by LDS-direct loads, as in the dQ kernel)
-//   phase 1: member m of a pair computes S, dP, P and dS of query block m (16 MFMA + softmax)
-//            and leaves P and dS, already packed as B operands, in an LDS exchange slot;
-//   phase 2: after a barrier each member accumulates, for BOTH query blocks, the half of the head
-//            dimension it owns: dV^T[2m..2m+1] += dO^T P, dK^T[2m..2m+1] += Q^T dS (16 MFMA).
+//   score step:        member m of a pair computes S, dP, P and dS of query block m (16 MFMA +
+//                      softmax) and leaves P and dS, already packed as B operands, in an LDS slot;
+//   accumulation step: each member accumulates, for BOTH query blocks, the half of the head
+//                      dimension it owns: dV^T[2m..2m+1] += dO^T P, dK^T[2m..2m+1] += Q^T dS (16 MFMA).
 // No MFMA is executed twice, and a wave keeps only 128 persistent registers.
 template <typename T, int D, bool CAUSAL, int MASK, bool DROPOUT>
 __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p) {
@@ -867,6 +618,11 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
         kf[kk] = *reinterpret_cast<const u32x4*>(kbase + static_cast<int64_t>(key) * p.ks[2] * 2 + (2 * kk + h) * 16);
         vf[kk] = *reinterpret_cast<const u32x4*>(vbase + static_cast<int64_t>(key) * p.vs[2] * 2 + (2 * kk + h) * 16);
     }
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+        settle(kf[kk]);
+        settle(vf[kk]);
+    }
     const float c = p.scale_log2;
 
     f32x16 dk[DH], dv[DH];
@@ -894,13 +650,12 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
             const char* tile_src = is_g ? gbase + static_cast<int64_t>(t) * kBN * grow_bytes
                                         : qbase + static_cast<int64_t>(t) * kBN * qrow_bytes;
             char* dst = stage + (is_g ? Tile::kBytes + (blk - Tile::kBlocks) * 1024 : blk * 1024);
-            __builtin_amdgcn_global_load_lds(TRI_GLB_PTR(tile_src + src_off[i]), TRI_LDS_PTR(dst), 16, 0, 0);
+            lds_direct_load16(tile_src + src_off[i], dst);
         }
         if (wave == 0)
-            __builtin_amdgcn_global_load_lds(TRI_GLB_PTR(lse_base + t * kBN + lane), TRI_LDS_PTR(stage + 2 * Tile::kBytes), 4, 0, 0);
+            lds_direct_load4(lse_base + t * kBN + lane, stage + 2 * Tile::kBytes);
         if (wave == NW - 1)
-            __builtin_amdgcn_global_load_lds(TRI_GLB_PTR(delta_base + t * kBN + lane),
-                                             TRI_LDS_PTR(stage + 2 * Tile::kBytes + kBN * 4), 4, 0, 0);
+            lds_direct_load4(delta_base + t * kBN + lane, stage + 2 * Tile::kBytes + kBN * 4);
     };
     issue_tile(t_begin);
     if (t_begin + 1 < n_tiles) issue_tile(t_begin + 1);
@@ -910,24 +665,39 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
     char* my_xch = xch + wave * 4096 + lane * 16;
     const char* peer_xch = xch + (wave ^ 4) * 4096 + lane * 16;
 
-    for (int j = t_begin; j < n_tiles; ++j) {
-        // tile j has landed (tile j+1 may still be in flight) and is visible; every wave is done with
-        // tile j-1 and with the exchange slots, so tile j+2 may overwrite the slot of tile j-1
-        if (j + 1 < n_tiles) TRI_WAIT_VMCNT(kLoadsPerTile);
+    // The two members of a pair sit on the same SIMD and run half a tile apart, so that one is in
+    // its score phase (softmax arithmetic) while the other is in its accumulation phase (MFMA only).
+    // Half-step hs: member 0 scores tile hs/2 on even steps, member 1 on odd steps; a wave publishes
+    // its P and dS at the start of its next accumulation step, so a slot is never rewritten before
+    // the barrier after the partner's read. Member 1 accumulates tile t on step 2t+2, member 0 on
+    // step 2t+3; by then it has scored tile t+1, so it takes its own P and dS of tile t back from
+    // its slot just before it overwrites them.
+    const int n_local = n_tiles - t_begin;
+    u32x4 cur_p[2], cur_s[2];
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+        cur_p[g] = cur_s[g] = u32x4{0, 0, 0, 0};
+        *reinterpret_cast<u32x4*>(my_xch + g * 1024) = cur_p[g];
+        *reinterpret_cast<u32x4*>(my_xch + (2 + g) * 1024) = cur_s[g];
+    }
+
+    // even half-step 2*lt: tile lt must have landed; tile lt+1 is the only other one that can be in
+    // flight. After the barrier every wave is done with tile lt-2, whose slot tile lt+1 takes.
+    auto open_even_step = [&](int lt) {
+        if (lt == 0 && n_local > 1) TRI_WAIT_VMCNT(kLoadsPerTile);
         else TRI_WAIT_VMCNT(0);
-        __syncthreads();
-        if (j + 2 < n_tiles) issue_tile(j + 2);
-
-        const char* sQ = smem + (j % kStages) * kStageBytes;
-        const char* sG = sQ + Tile::kBytes;
-        const float* sLse = reinterpret_cast<const float*>(sG + Tile::kBytes);
-        const float* sDelta = sLse + kBN;
-        const int r0 = j * kBN;
-        const int rb = r0 + 32 * member;  // first row of the query block this wave scores
-
-        // ---- phase 1: P and dS of query block `member` against this pair's keys
-        u32x4 pb[2], sb[2];
-        if (!CAUSAL || rb + 31 >= wkey0) {
+        lds_barrier();
+        if (lt >= 1 && lt + 1 < n_local) issue_tile(t_begin + lt + 1);
+    };
+    // score step: P and dS of query block `member` of local tile lt against this pair's keys
+    auto score = [&](int lt) {
+        const int j = t_begin + lt;
+        const int rb = j * kBN + 32 * member;
+        if (lt < n_local && (!CAUSAL || rb + 31 >= wkey0)) {
+            const char* sQ = smem + (j % kStages) * kStageBytes;
+            const char* sG = sQ + Tile::kBytes;
+            const float* sLse = reinterpret_cast<const float*>(sG + Tile::kBytes);
+            const float* sDelta = sLse + kBN;
             const bool diag = CAUSAL && rb < wkey0 + 31;
             float mk[MASK != kNoMask ? 16 : 1];
             if constexpr (MASK != kNoMask) {
@@ -937,71 +707,93 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
                     mk[i] = mask_at<T, MASK>(p.mask, mbase + static_cast<int64_t>(rb + c_row(i, h)) * p.ms[2]);
             }
             const int qoff = 32 * member * Tile::kRowBytes;
-            u32x4 fr[KK];
+            // row fragments of Q, then of dO, through a ring of kRing reads in flight
+            constexpr int kRing = 4;
+            auto row_frag = [&](int n) {
+                return lds_read16(n < KK ? sQ : sG, (row_off0 ^ ((n % KK) << 5)) + qoff);
+            };
+            u32x4 fr[kRing];
 #pragma unroll
-            for (int kk = 0; kk < KK; ++kk) fr[kk] = lds_read16(sQ, (row_off0 ^ (kk << 5)) + qoff);
+            for (int n = 0; n < kRing; ++n) fr[n] = row_frag(n);
             __builtin_amdgcn_sched_barrier(0);
             f32x16 s = zero16(), dp = zero16();
 #pragma unroll
-            for (int kk = 0; kk < KK; ++kk) {
-                s = Mma<T>::run(fr[kk], kf[kk], s);
-                fr[kk] = lds_read16(sG, (row_off0 ^ (kk << 5)) + qoff);
+            for (int n = 0; n < 2 * KK; ++n) {
+                if (n < KK) s = Mma<T>::run(fr[n % kRing], kf[n], s);
+                else dp = Mma<T>::run(fr[n % kRing], vf[n - KK], dp);
+                if (n + kRing < 2 * KK) fr[n % kRing] = row_frag(n + kRing);
                 __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
-            for (int kk = 0; kk < KK; ++kk) dp = Mma<T>::run(fr[kk], vf[kk], dp);
-            __builtin_amdgcn_sched_barrier(0);
-            float pr[16], ds[16];
+            for (int gg = 0; gg < 2; ++gg) {  // eight rows at a time, packed as soon as they are done
+                float pr[8], ds[8];
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + 32 * member + 8 * g + 4 * h);
-                const f32x4 d4 = *reinterpret_cast<const f32x4*>(sDelta + 32 * member + 8 * g + 4 * h);
-                if constexpr (MASK != kNoMask) {
+                for (int g2 = 0; g2 < 2; ++g2) {
+                    const int g = 2 * gg + g2;
+                    f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + 32 * member + 8 * g + 4 * h);
+                    const f32x4 d4 = *reinterpret_cast<const f32x4*>(sDelta + 32 * member + 8 * g + 4 * h);
+                    if constexpr (MASK != kNoMask) {
 #pragma unroll
-                    for (int bb = 0; bb < 4; ++bb) l4[bb] = l4[bb] == -INFINITY ? INFINITY : l4[bb];
-                }
-                uint32_t dw[4];
-                if constexpr (DROPOUT) {
-                    const Philox4 r = dropout_block(p, bh, (rb + 8 * g + 4 * h) >> 2, key >> 2);
-#pragma unroll
-                    for (int bb = 0; bb < 4; ++bb) dw[bb] = (r.w[bb] >> (8 * (key & 3))) & 0xffu;
-                }
-#pragma unroll
-                for (int bb = 0; bb < 4; ++bb) {
-                    const int i = 4 * g + bb;
-                    float pv;
-                    if constexpr (MASK != kNoMask) pv = fast_exp2(fmaf(mk[i], kLog2e, s[i] * c) - l4[bb]);
-                    else pv = fast_exp2(fmaf(s[i], c, -l4[bb]));
-                    if (diag) pv = key <= rb + c_row(i, h) ? pv : 0.f;
-                    float dpv = dp[i];
-                    if constexpr (DROPOUT) {
-                        const bool keep = static_cast<int>(dw[bb]) >= p.thr8;
-                        dpv = keep ? dpv * p.zscale : 0.f;
-                        pr[i] = keep ? pv * p.zscale : 0.f;
-                    } else {
-                        pr[i] = pv;
+                        for (int bb = 0; bb < 4; ++bb) l4[bb] = l4[bb] == -INFINITY ? INFINITY : l4[bb];
                     }
-                    ds[i] = pv * (dpv - d4[bb]);
-                }
-            }
+                    uint32_t dw[4];
+                    if constexpr (DROPOUT) {
+                        const Philox4 r = dropout_block(p, bh, (rb + 8 * g + 4 * h) >> 2, key >> 2);
 #pragma unroll
-            for (int g = 0; g < 2; ++g) {
-                pb[g] = pack8<T>(&pr[8 * g]);
-                sb[g] = pack8<T>(&ds[8 * g]);
+                        for (int bb = 0; bb < 4; ++bb) dw[bb] = (r.w[bb] >> (8 * (key & 3))) & 0xffu;
+                    }
+#pragma unroll
+                    for (int bb = 0; bb < 4; ++bb) {
+                        const int i = 4 * g + bb;
+                        float pv;
+                        if constexpr (MASK != kNoMask) pv = fast_exp2(fmaf(mk[i], kLog2e, s[i] * c) - l4[bb]);
+                        else pv = fast_exp2(fmaf(s[i], c, -l4[bb]));
+                        if (diag) pv = key <= rb + c_row(i, h) ? pv : 0.f;
+                        float dpv = dp[i];
+                        if constexpr (DROPOUT) {
+                            const bool keep = static_cast<int>(dw[bb]) >= p.thr8;
+                            dpv = keep ? dpv * p.zscale : 0.f;
+                            pr[4 * g2 + bb] = keep ? pv * p.zscale : 0.f;
+                        } else {
+                            pr[4 * g2 + bb] = pv;
+                        }
+                        ds[4 * g2 + bb] = pv * (dpv - d4[bb]);
+                    }
+                }
+                cur_p[gg] = pack8<T>(pr);
+                cur_s[gg] = pack8<T>(ds);
+                __builtin_amdgcn_sched_barrier(0);
             }
         } else {
 #pragma unroll
-            for (int g = 0; g < 2; ++g) pb[g] = sb[g] = u32x4{0, 0, 0, 0};
+            for (int g = 0; g < 2; ++g) cur_p[g] = cur_s[g] = u32x4{0, 0, 0, 0};
         }
+    };
+    // accumulation step: publish the latest scores, then add local tile lt to this member's half of
+    // the head dimension for both query blocks
+    auto accumulate = [&](int lt) {
+        u32x4 own_p[2], own_s[2];
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
-            *reinterpret_cast<u32x4*>(my_xch + g * 1024) = pb[g];
-            *reinterpret_cast<u32x4*>(my_xch + (2 + g) * 1024) = sb[g];
+            if (member == 0) {  // LDS operations of one wave complete in order: read, then overwrite
+                own_p[g] = *reinterpret_cast<const u32x4*>(my_xch + g * 1024);
+                own_s[g] = *reinterpret_cast<const u32x4*>(my_xch + (2 + g) * 1024);
+            } else {
+                own_p[g] = cur_p[g];
+                own_s[g] = cur_s[g];
+            }
         }
-        __syncthreads();
-
-        // ---- phase 2: this member's half of the head dimension, both query blocks
-        if (!CAUSAL || r0 + kBN - 1 >= wkey0) {
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            *reinterpret_cast<u32x4*>(my_xch + g * 1024) = cur_p[g];
+            *reinterpret_cast<u32x4*>(my_xch + (2 + g) * 1024) = cur_s[g];
+        }
+        const int j = t_begin + lt;
+        const int r0 = j * kBN;
+        if (lt >= 0 && lt < n_local && (!CAUSAL || r0 + kBN - 1 >= wkey0)) {
+            const char* sQ = smem + (j % kStages) * kStageBytes;
+            const char* sG = sQ + Tile::kBytes;
             u32x4 pp[2], ps[2];  // the partner's P and dS
 #pragma unroll
             for (int g = 0; g < 2; ++g) {
@@ -1012,8 +804,8 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
             for (int qb = 0; qb < 2; ++qb) {
 #pragma unroll
                 for (int g = 0; g < 2; ++g) {
-                    const u32x4 bp = qb == member ? pb[g] : pp[g];
-                    const u32x4 bs = qb == member ? sb[g] : ps[g];
+                    const u32x4 bp = qb == member ? own_p[g] : pp[g];
+                    const u32x4 bs = qb == member ? own_s[g] : ps[g];
                     u32x4 tf[DH];
 #pragma unroll
                     for (int d = 0; d < DH; ++d) {
@@ -1028,8 +820,27 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
                     }
 #pragma unroll
                     for (int d = 0; d < DH; ++d) dk[d] = Mma<T>::run(tf[d], bs, dk[d]);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
+        }
+    };
+
+    if (member == 0) {
+#pragma unroll 1
+        for (int lt = 0; lt <= n_local; ++lt) {
+            open_even_step(lt);
+            score(lt);
+            lds_barrier();
+            accumulate(lt - 1);
+        }
+    } else {
+#pragma unroll 1
+        for (int lt = 0; lt <= n_local; ++lt) {
+            open_even_step(lt);
+            accumulate(lt - 1);
+            lds_barrier();
+            score(lt);
         }
     }
 
@@ -1084,7 +895,7 @@ int launch_dkdv_dropout(const KParams& p, hipStream_t stream) {
         return launch_dkdv_waves<T, D, 4, CAUSAL, MASK>(p, stream);
     } else {
         // D = 128: K, V and both gradient accumulators of a 32-key block take 192 registers, too many
-        // for two waves per SIMD; the one-wave pipelined kernel serves the plain and causal variants,
+        // for two waves per SIMD, so the plain and causal variants pair two waves on each key block;
         // the mask and dropout variants (which need still more registers) keep the staged kernel
         const dim3 grid(p.B * p.H * (p.S / kBM)), block(256);
         if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, CAUSAL, MASK, true>), grid, block, 0, stream, p);

@@ -144,6 +144,30 @@ __device__ __forceinline__ void lds_write8(char* smem, int off, u32x2 v) { *rein
 #define TRI_GLB_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
+// LDS-direct loads and the matching barrier, issued through inline assembly. The compiler's own
+// intrinsic for these loads is correct but pessimistic: it cannot tell which LDS reads depend on
+// a load in flight, so it drains the vector-memory counter before the next LDS read and before
+// every __syncthreads(), which turns a prefetch several tiles deep into a synchronous copy.
+// Kernels that use these helpers order the loads themselves: TRI_WAIT_VMCNT(n) for "all but the
+// last n loads have landed", then lds_barrier() to make them (and ordinary LDS writes) visible
+// to the other waves. `lds_dst` must be uniform across the wave; lane l's 16 (4) bytes land at
+// lds_dst + 16*l (4*l). M0 holds the LDS address and needs one wait state before the load.
+__device__ __forceinline__ void lds_direct_load16(const void* src, const void* lds_dst) {
+    const uint32_t dst = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(TRI_LDS_PTR(lds_dst))));
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(dst), "v"(src) : "memory", "m0");
+}
+__device__ __forceinline__ void lds_direct_load4(const void* src, const void* lds_dst) {
+    const uint32_t dst = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(TRI_LDS_PTR(lds_dst))));
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(dst), "v"(src) : "memory", "m0");
+}
+// Makes the compiler wait HERE for a value that an earlier global load produces. Otherwise the
+// wait lands at the first use, which may be inside a loop that keeps LDS-direct loads in flight;
+// the compiler does not know about those and its wait would drain them on every iteration.
+template <typename V>
+__device__ __forceinline__ void settle(const V& v) { asm volatile("" : : "v"(v)); }
+// Workgroup barrier that waits for this wave's LDS traffic only, not for loads still in flight.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : : : "memory"); }
+
 template <int D>
 struct SwzTile {
     static constexpr int kRowBytes = D * 2;
@@ -166,7 +190,7 @@ struct SwzTile {
         return row * row_stride_bytes + c * 16;
     }
     static __device__ __forceinline__ void load_block(char* tile, int blk, const char* src) {
-        __builtin_amdgcn_global_load_lds(TRI_GLB_PTR(src), TRI_LDS_PTR(tile + blk * 1024), 16, 0, 0);
+        lds_direct_load16(src, tile + blk * 1024);
     }
     // byte offset (within the tile) a lane passes to the transposed read of column block db
     // (32 columns), half = 0/1 (K-slots 0-3 / 4-7); add ks * 16 * kRowBytes for K-step ks
