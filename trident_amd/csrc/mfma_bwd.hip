@@ -2,10 +2,10 @@
 // (replaces trident/kernel/attention.py:169-339, split in two passes so that no gradient
 // tile is ever accumulated in global memory):
 //
-//   dQ pass    one workgroup per 128 query rows (a wave owns 32), streaming key tiles of 64:
+//   dQ pass    one workgroup per 256 (128) query rows (a wave owns 32), streaming key tiles of 64:
 //              S^T = K Q^T, dP^T = V dO^T, dS^T = P^T * (dP^T - delta), dQ^T += K^T dS^T
-//   dK/dV pass one workgroup per 128 keys (a wave owns 32), streaming query tiles of 64:
-//              S = Q K^T, dP = dO V^T, dV^T += dO^T P, dK^T += Q^T dS
+//   dK/dV pass one workgroup per 256 (128) keys (a wave, or for D = 128 a pair of waves, owns 32),
+//              streaming query tiles of 64: S = Q K^T, dP = dO V^T, dV^T += dO^T P, dK^T += Q^T dS
 //
 // In both, the lane index is the row that owns the accumulators (query row resp. key), the
 // stationary operands (Q,dO resp. K,V) stay in registers as MFMA B operands, and P / dS go
@@ -102,7 +102,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
             const bool is_v = blk >= Tile::kBlocks;
             const char* tile_src = is_v ? vbase + static_cast<int64_t>(t) * kBN * vrow_bytes
                                         : kbase + static_cast<int64_t>(t) * kBN * krow_bytes;
-            lds_direct_load16(tile_src + src_off[i], stage + blk * 1024);
+            lds_direct_load16(tile_src, src_off[i], stage + blk * 1024);
         }
     };
     issue_tile(0);
@@ -199,164 +199,6 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
         }
 }
 
-// --------------------------------------------------------------------------------- dK, dV
-template <typename T, int D, bool CAUSAL, int MASK, bool DROPOUT>
-__global__ __launch_bounds__(256, 2) void mfma_dkdv_kernel(const KParams p) {
-    constexpr int kRowBytes = RowTile<D>::bytes(kBN);
-    constexpr int kTransBytes = TransTile::bytes(D);
-    constexpr int KK = D / 16;
-    constexpr int DB = D / 32;
-    __shared__ __attribute__((aligned(16))) char smem[2 * kRowBytes + 2 * kTransBytes + 2 * kBN * 4];
-    char* sQ = smem;
-    char* sG = smem + kRowBytes;
-    char* sQt = smem + 2 * kRowBytes;
-    char* sGt = sQt + kTransBytes;
-    float* sLse = reinterpret_cast<float*>(sGt + kTransBytes);
-    float* sDelta = sLse + kBN;
-
-    const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
-    int bh, kt;
-    map_block(blockIdx.x, p.B * p.H, p.S / kBM, CAUSAL ? kHeavyFirst : kUniformTiles, &bh, &kt);
-    const int b = bh / p.H, hd = bh % p.H;
-    const int k0 = kt * kBM;
-    const int wkey0 = k0 + 32 * wave;
-    const int key = wkey0 + l32;
-
-    const char* krowp = static_cast<const char*>(p.k) + (b * p.ks[0] + hd * p.ks[1] + static_cast<int64_t>(key) * p.ks[2]) * 2;
-    const char* vrowp = static_cast<const char*>(p.v) + (b * p.vs[0] + hd * p.vs[1] + static_cast<int64_t>(key) * p.vs[2]) * 2;
-    const char* qbase = static_cast<const char*>(p.q) + (b * p.qs[0] + hd * p.qs[1]) * 2;
-    const char* gbase = static_cast<const char*>(p.d_o) + (b * p.dos[0] + hd * p.dos[1]) * 2;
-    const int64_t qrow_bytes = p.qs[2] * 2, grow_bytes = p.dos[2] * 2;
-    const float* lse_base = p.lse + static_cast<int64_t>(bh) * p.S;
-    const float* delta_base = p.delta + static_cast<int64_t>(bh) * p.S;
-
-    u32x4 kf[KK], vf[KK];
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-        kf[kk] = *reinterpret_cast<const u32x4*>(krowp + (2 * kk + h) * 16);
-        vf[kk] = *reinterpret_cast<const u32x4*>(vrowp + (2 * kk + h) * 16);
-    }
-    const float c = p.scale_log2;
-
-    f32x16 dk[DB], dv[DB];
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-        dk[db] = zero16();
-        dv[db] = zero16();
-    }
-
-    const int j_begin = CAUSAL ? k0 / kBN : 0;
-    const int n_tiles = p.S / kBN;
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): K/V fragments are in registers
-    for (int j = j_begin; j < n_tiles; ++j) {
-        const int r0 = j * kBN;
-        {
-            uint32_t st[StageRegs<D>::kCount];
-            TransStage<D>::load(st, qbase + r0 * qrow_bytes, qrow_bytes, tid);
-            TransStage<D>::store_rows(st, sQ, tid);
-            TransStage<D>::store(st, sQt, tid);
-            TransStage<D>::load(st, gbase + r0 * grow_bytes, grow_bytes, tid);
-            TransStage<D>::store_rows(st, sG, tid);
-            TransStage<D>::store(st, sGt, tid);
-            if (tid < kBN) {
-                float l = lse_base[r0 + tid];
-                sLse[tid] = l == -INFINITY ? INFINITY : l;
-                sDelta[tid] = delta_base[r0 + tid];
-            }
-        }
-        __syncthreads();
-        const bool active = !CAUSAL || r0 + kBN - 1 >= wkey0;
-        if (active) {
-#pragma unroll
-            for (int qb = 0; qb < 2; ++qb) {
-                const int rb = r0 + 32 * qb;  // first query row of this block
-                if (CAUSAL && rb + 31 < wkey0) continue;
-                const bool diag = CAUSAL && rb < wkey0 + 31;
-                float mk[MASK != kNoMask ? 16 : 1];
-                if constexpr (MASK != kNoMask) {
-                    const int64_t mbase = b * p.ms[0] + hd * p.ms[1] + key;
-#pragma unroll
-                    for (int i = 0; i < 16; ++i)
-                        mk[i] = mask_at<T, MASK>(p.mask, mbase + static_cast<int64_t>(rb + c_row(i, h)) * p.ms[2]);
-                }
-                f32x16 s = zero16(), dp = zero16();
-#pragma unroll
-                for (int kk = 0; kk < KK; ++kk) {
-                    const u32x4 a = lds_read16(sQ, RowTile<D>::off(32 * qb + l32, 2 * kk + h));
-                    s = Mma<T>::run(a, kf[kk], s);
-                }
-#pragma unroll
-                for (int kk = 0; kk < KK; ++kk) {
-                    const u32x4 a = lds_read16(sG, RowTile<D>::off(32 * qb + l32, 2 * kk + h));
-                    dp = Mma<T>::run(a, vf[kk], dp);
-                }
-                float pr[16], ds[16];
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + 32 * qb + 8 * g + 4 * h);
-                    const f32x4 d4 = *reinterpret_cast<const f32x4*>(sDelta + 32 * qb + 8 * g + 4 * h);
-                    uint32_t dw[4];
-                    if constexpr (DROPOUT) {
-                        const Philox4 r = dropout_block(p, bh, (rb + 8 * g + 4 * h) >> 2, key >> 2);
-#pragma unroll
-                        for (int bb = 0; bb < 4; ++bb) dw[bb] = (r.w[bb] >> (8 * (key & 3))) & 0xffu;
-                    }
-#pragma unroll
-                    for (int bb = 0; bb < 4; ++bb) {
-                        const int i = 4 * g + bb;
-                        const int qrow = rb + c_row(i, h);
-                        float x = s[i] * c;
-                        if constexpr (MASK != kNoMask) x = fmaf(mk[i], kLog2e, x);
-                        float pv = fast_exp2(x - l4[bb]);
-                        if (diag) pv = key <= qrow ? pv : 0.f;
-                        float dpv = dp[i];
-                        if constexpr (DROPOUT) {
-                            const bool keep = static_cast<int>(dw[bb]) >= p.thr8;
-                            dpv = keep ? dpv * p.zscale : 0.f;
-                            pr[i] = keep ? pv * p.zscale : 0.f;
-                        } else {
-                            pr[i] = pv;
-                        }
-                        ds[i] = pv * (dpv - d4[bb]);
-                    }
-                }
-#pragma unroll
-                for (int g = 0; g < 2; ++g) {
-                    const u32x4 pb = pack8<T>(&pr[8 * g]);
-                    const u32x4 sb = pack8<T>(&ds[8 * g]);
-#pragma unroll
-                    for (int db = 0; db < DB; ++db) {
-                        const u32x4 a = lds_read16(sGt, TransTile::read_off(32 * db + l32, 2 * qb + g, h));
-                        dv[db] = Mma<T>::run(a, pb, dv[db]);
-                    }
-#pragma unroll
-                    for (int db = 0; db < DB; ++db) {
-                        const u32x4 a = lds_read16(sQt, TransTile::read_off(32 * db + l32, 2 * qb + g, h));
-                        dk[db] = Mma<T>::run(a, sb, dk[db]);
-                    }
-                }
-            }
-        }
-        __syncthreads();
-    }
-
-    char* dkrow = static_cast<char*>(p.dk) + (b * p.dks[0] + hd * p.dks[1] + static_cast<int64_t>(key) * p.dks[2]) * 2;
-    char* dvrow = static_cast<char*>(p.dv) + (b * p.dvs[0] + hd * p.dvs[1] + static_cast<int64_t>(key) * p.dvs[2]) * 2;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            u32x2 a, e;
-            a.x = Mma<T>::pack2(dk[db][4 * g + 0] * p.scale, dk[db][4 * g + 1] * p.scale);
-            a.y = Mma<T>::pack2(dk[db][4 * g + 2] * p.scale, dk[db][4 * g + 3] * p.scale);
-            e.x = Mma<T>::pack2(dv[db][4 * g + 0], dv[db][4 * g + 1]);
-            e.y = Mma<T>::pack2(dv[db][4 * g + 2], dv[db][4 * g + 3]);
-            *reinterpret_cast<u32x2*>(dkrow + (32 * db + 8 * g + 4 * h) * 2) = a;
-            *reinterpret_cast<u32x2*>(dvrow + (32 * db + 8 * g + 4 * h) * 2) = e;
-        }
-}
-
 // ------------------------------------------------------------------ dK, dV (8 waves)
 // Same data flow as the dQ kernel with the roles of queries and keys exchanged: a workgroup of
 // NW waves owns 32*NW keys, one wave 32 of them with its K and V rows in registers (B operands)
@@ -434,12 +276,12 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
             const char* tile_src = is_g ? gbase + static_cast<int64_t>(t) * kBN * grow_bytes
                                         : qbase + static_cast<int64_t>(t) * kBN * qrow_bytes;
             char* dst = stage + (is_g ? Tile::kBytes + (blk - Tile::kBlocks) * 1024 : blk * 1024);
-            lds_direct_load16(tile_src + src_off[i], dst);
+            lds_direct_load16(tile_src, src_off[i], dst);
         }
         if (wave == 0)
-            lds_direct_load4(lse_base + t * kBN + lane, stage + 2 * Tile::kBytes);
+            lds_direct_load4(lse_base + t * kBN, lane * 4, stage + 2 * Tile::kBytes);
         if (wave == NW - 1)
-            lds_direct_load4(delta_base + t * kBN + lane, stage + 2 * Tile::kBytes + kBN * 4);
+            lds_direct_load4(delta_base + t * kBN, lane * 4, stage + 2 * Tile::kBytes + kBN * 4);
     };
     issue_tile(t_begin);
     if (t_begin + 1 < n_tiles) issue_tile(t_begin + 1);
@@ -650,12 +492,12 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
             const char* tile_src = is_g ? gbase + static_cast<int64_t>(t) * kBN * grow_bytes
                                         : qbase + static_cast<int64_t>(t) * kBN * qrow_bytes;
             char* dst = stage + (is_g ? Tile::kBytes + (blk - Tile::kBlocks) * 1024 : blk * 1024);
-            lds_direct_load16(tile_src + src_off[i], dst);
+            lds_direct_load16(tile_src, src_off[i], dst);
         }
         if (wave == 0)
-            lds_direct_load4(lse_base + t * kBN + lane, stage + 2 * Tile::kBytes);
+            lds_direct_load4(lse_base + t * kBN, lane * 4, stage + 2 * Tile::kBytes);
         if (wave == NW - 1)
-            lds_direct_load4(delta_base + t * kBN + lane, stage + 2 * Tile::kBytes + kBN * 4);
+            lds_direct_load4(delta_base + t * kBN, lane * 4, stage + 2 * Tile::kBytes + kBN * 4);
     };
     issue_tile(t_begin);
     if (t_begin + 1 < n_tiles) issue_tile(t_begin + 1);
@@ -895,12 +737,10 @@ int launch_dkdv_dropout(const KParams& p, hipStream_t stream) {
         return launch_dkdv_waves<T, D, 4, CAUSAL, MASK>(p, stream);
     } else {
         // D = 128: K, V and both gradient accumulators of a 32-key block take 192 registers, too many
-        // for two waves per SIMD, so the plain and causal variants pair two waves on each key block;
-        // the mask and dropout variants (which need still more registers) keep the staged kernel
-        const dim3 grid(p.B * p.H * (p.S / kBM)), block(256);
-        if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, CAUSAL, MASK, true>), grid, block, 0, stream, p);
-        else if (MASK != kNoMask) hipLaunchKernelGGL((mfma_dkdv_kernel<T, D, CAUSAL, MASK, false>), grid, block, 0, stream, p);
-        else hipLaunchKernelGGL((mfma_dkdv_pair_kernel<T, D, CAUSAL, kNoMask, false>), grid, dim3(512), 0, stream, p);
+        // for two waves per SIMD, so two waves are paired on each key block of a 128-key workgroup
+        const dim3 grid(p.B * p.H * (p.S / kBM)), block(512);
+        if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dkdv_pair_kernel<T, D, CAUSAL, MASK, true>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((mfma_dkdv_pair_kernel<T, D, CAUSAL, MASK, false>), grid, block, 0, stream, p);
         return static_cast<int>(hipGetLastError());
     }
 }

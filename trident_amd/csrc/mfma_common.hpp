@@ -150,15 +150,16 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 // every __syncthreads(), which turns a prefetch several tiles deep into a synchronous copy.
 // Kernels that use these helpers order the loads themselves: TRI_WAIT_VMCNT(n) for "all but the
 // last n loads have landed", then lds_barrier() to make them (and ordinary LDS writes) visible
-// to the other waves. `lds_dst` must be uniform across the wave; lane l's 16 (4) bytes land at
-// lds_dst + 16*l (4*l). M0 holds the LDS address and needs one wait state before the load.
-__device__ __forceinline__ void lds_direct_load16(const void* src, const void* lds_dst) {
+// to the other waves. `base` and `lds_dst` must be uniform across the wave (they travel in scalar
+// registers); a lane reads at base + lane_off (unsigned 32-bit byte offset) and its 16 (4) bytes
+// land at lds_dst + 16*l (4*l). M0 holds the LDS address and needs one wait state before the load.
+__device__ __forceinline__ void lds_direct_load16(const void* base, uint32_t lane_off, const void* lds_dst) {
     const uint32_t dst = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(TRI_LDS_PTR(lds_dst))));
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(dst), "v"(src) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(lane_off), "s"(base) : "memory", "m0");
 }
-__device__ __forceinline__ void lds_direct_load4(const void* src, const void* lds_dst) {
+__device__ __forceinline__ void lds_direct_load4(const void* base, uint32_t lane_off, const void* lds_dst) {
     const uint32_t dst = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(TRI_LDS_PTR(lds_dst))));
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(dst), "v"(src) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" : : "s"(dst), "v"(lane_off), "s"(base) : "memory", "m0");
 }
 // Makes the compiler wait HERE for a value that an earlier global load produces. Otherwise the
 // wait lands at the first use, which may be inside a loop that keeps LDS-direct loads in flight;
@@ -188,9 +189,6 @@ struct SwzTile {
         const int row = blk * kRowsPerBlock + lane / kChunks;
         const int c = (lane % kChunks) ^ swz(row);
         return row * row_stride_bytes + c * 16;
-    }
-    static __device__ __forceinline__ void load_block(char* tile, int blk, const char* src) {
-        lds_direct_load16(src, tile + blk * 1024);
     }
     // byte offset (within the tile) a lane passes to the transposed read of column block db
     // (32 columns), half = 0/1 (K-slots 0-3 / 4-7); add ks * 16 * kRowBytes for K-step ks

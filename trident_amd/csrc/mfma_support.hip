@@ -47,6 +47,9 @@ int launch_delta_t(const KParams& p, hipStream_t stream) {
 
 }  // namespace
 
+// 64 rows of a tile must be reachable with an unsigned 32-bit byte offset (2-byte elements)
+static bool tile_offsets_fit(const int64_t* strides) { return strides[2] >= 0 && strides[2] < (int64_t{1} << 24); }
+
 bool mfma_supported(int which, int dtype, const KParams& p) {
     if (dtype != TRI_ATTN_F16 && dtype != TRI_ATTN_BF16) return false;
     if (p.D != 64 && p.D != 128) return false;
@@ -63,9 +66,12 @@ bool mfma_supported(int which, int dtype, const KParams& p) {
         case kMfmaFwd:
             return aligned16(p.o) && strides8(p.os);
         case kMfmaDkdv:
+            // the streamed tiles are addressed with 32-bit byte offsets from a per-tile base
+            if (!tile_offsets_fit(p.qs) || !tile_offsets_fit(p.dos)) return false;
             return aligned16(p.d_o) && strides8(p.dos) && aligned16(p.dk) && strides8(p.dks) && aligned16(p.dv) &&
                    strides8(p.dvs);
         case kMfmaDq:
+            if (!tile_offsets_fit(p.ks) || !tile_offsets_fit(p.vs)) return false;
             // the mask gradient is written by the generic dQ kernel
             return p.dmask == nullptr && aligned16(p.d_o) && strides8(p.dos) && aligned16(p.dq) && strides8(p.dqs);
         default:
