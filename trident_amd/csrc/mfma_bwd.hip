@@ -50,7 +50,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63, l32 = lane & 31, h = lane >> 5;
     int bh, qt;
-    map_block(blockIdx.x, p.B * p.H, p.S / kRows, CAUSAL ? kHeavyLast : kUniformTiles, &bh, &qt);
+    map_block_for<MASK>(p, blockIdx.x, p.S / kRows, CAUSAL ? kHeavyLast : kUniformTiles, &bh, &qt);
     const int b = bh / p.H, hd = bh % p.H;
     const int q0 = qt * kRows;
     const int wrow0 = q0 + 32 * wave;
@@ -166,15 +166,16 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
                 ds[i] = pr;
             }
             if constexpr (DROPOUT) {
+                const Philox4 mine = dropout_block(p, bh, qrow >> 2, (t0 + 32 * kb + 8 * (lane & 3) + 4 * h) >> 2);
+                uint32_t w[4];
+                quad_row_words(mine, lane, w);
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const uint32_t w = dropout_word(p, bh, qrow, t0 + 32 * kb + 8 * g + 4 * h);
+                for (int g = 0; g < 4; ++g)
 #pragma unroll
                     for (int bb = 0; bb < 4; ++bb) {
-                        const bool keep = static_cast<int>((w >> (8 * bb)) & 0xffu) >= p.thr8;
+                        const bool keep = static_cast<int>((w[g] >> (8 * bb)) & 0xffu) >= p.thr8;
                         dpt[4 * g + bb] = keep ? dpt[4 * g + bb] * p.zscale : 0.f;
                     }
-                }
             }
 #pragma unroll
             for (int i = 0; i < 16; ++i) ds[i] *= dpt[i] - dlt;
@@ -223,7 +224,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63, l32 = lane & 31, h = lane >> 5;
     int bh, kt;
-    map_block(blockIdx.x, p.B * p.H, p.S / kKeys, CAUSAL ? kHeavyFirst : kUniformTiles, &bh, &kt);
+    map_block_for<MASK>(p, blockIdx.x, p.S / kKeys, CAUSAL ? kHeavyFirst : kUniformTiles, &bh, &kt);
     const int b = bh / p.H, hd = bh % p.H;
     const int k0 = kt * kKeys;
     const int wkey0 = k0 + 32 * wave;
@@ -336,6 +337,8 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
             u32x4 pb[2], sb[2];
             {
                 float pr[16], ds[16];
+                Philox4 mine;  // the block of rows rb + 8 (lane % 4) + 4 h .. +3: this lane's share of the quad's four
+                if constexpr (DROPOUT) mine = dropout_block(p, bh, (rb + 8 * (lane & 3) + 4 * h) >> 2, key >> 2);
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + 32 * qb + 8 * g + 4 * h);
@@ -346,7 +349,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
                     }
                     uint32_t dw[4];
                     if constexpr (DROPOUT) {
-                        const Philox4 r = dropout_block(p, bh, (rb + 8 * g + 4 * h) >> 2, key >> 2);
+                        const Philox4 r = quad_bcast_from(g, mine);  // lane g of the quad generated rows rb + 8 g + 4 h .. +3
 #pragma unroll
                         for (int bb = 0; bb < 4; ++bb) dw[bb] = (r.w[bb] >> (8 * (key & 3))) & 0xffu;
                     }
@@ -440,7 +443,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
     const int kb = wave & 3, member = wave >> 2;
     const int lane = tid & 63, l32 = lane & 31, h = lane >> 5;
     int bh, kt;
-    map_block(blockIdx.x, p.B * p.H, p.S / kKeys, CAUSAL ? kHeavyFirst : kUniformTiles, &bh, &kt);
+    map_block_for<MASK>(p, blockIdx.x, p.S / kKeys, CAUSAL ? kHeavyFirst : kUniformTiles, &bh, &kt);
     const int b = bh / p.H, hd = bh % p.H;
     const int k0 = kt * kKeys;
     const int wkey0 = k0 + 32 * kb;
@@ -566,6 +569,8 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
                 if (n + kRing < 2 * KK) fr[n % kRing] = row_frag(n + kRing);
                 __builtin_amdgcn_sched_barrier(0);
             }
+            Philox4 mine;  // the block of rows rb + 8 (lane % 4) + 4 h .. +3: this lane's share of the quad's four
+            if constexpr (DROPOUT) mine = dropout_block(p, bh, (rb + 8 * (lane & 3) + 4 * h) >> 2, key >> 2);
 #pragma unroll
             for (int gg = 0; gg < 2; ++gg) {  // eight rows at a time, packed as soon as they are done
                 float pr[8], ds[8];
@@ -580,7 +585,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
                     }
                     uint32_t dw[4];
                     if constexpr (DROPOUT) {
-                        const Philox4 r = dropout_block(p, bh, (rb + 8 * g + 4 * h) >> 2, key >> 2);
+                        const Philox4 r = quad_bcast_from(g, mine);  // lane g of the quad generated rows rb + 8 g + 4 h .. +3
 #pragma unroll
                         for (int bb = 0; bb < 4; ++bb) dw[bb] = (r.w[bb] >> (8 * (key & 3))) & 0xffu;
                     }

@@ -153,12 +153,15 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 // to the other waves. `base` and `lds_dst` must be uniform across the wave (they travel in scalar
 // registers); a lane reads at base + lane_off (unsigned 32-bit byte offset) and its 16 (4) bytes
 // land at lds_dst + 16*l (4*l). M0 holds the LDS address and needs one wait state before the load.
+// LDS byte address of a pointer into __shared__ memory: the shared aperture is 4 GiB aligned, so the
+// low half of the generic address is the LDS offset (no address-space cast, hence no null check).
+__device__ __forceinline__ uint32_t lds_address(const void* p) { return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p)); }
 __device__ __forceinline__ void lds_direct_load16(const void* base, uint32_t lane_off, const void* lds_dst) {
-    const uint32_t dst = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(TRI_LDS_PTR(lds_dst))));
+    const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_address(lds_dst));
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(lane_off), "s"(base) : "memory", "m0");
 }
 __device__ __forceinline__ void lds_direct_load4(const void* base, uint32_t lane_off, const void* lds_dst) {
-    const uint32_t dst = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(TRI_LDS_PTR(lds_dst))));
+    const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_address(lds_dst));
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" : : "s"(dst), "v"(lane_off), "s"(base) : "memory", "m0");
 }
 // Makes the compiler wait HERE for a value that an earlier global load produces. Otherwise the
@@ -339,6 +342,65 @@ __device__ __forceinline__ void map_block(int bid, int num_heads, int num_tiles,
     }
     *bh = head;
     *tile = heavy_last ? num_tiles - 1 - t : t;
+}
+
+// Mapping for a mask that is shared by the H heads of a batch (head stride 0). The mask, not K/V,
+// is then the big stream (S*S*4 bytes per batch against 4*S*D per head), so the H workgroups that
+// read the same mask tile get consecutive slots of ONE XCD: they run side by side, the first one
+// pulls the tile from HBM and the others find it in that XCD's L2.
+__device__ __forceinline__ void map_block_shared_mask(int bid, int batches, int heads, int num_tiles, int* bh, int* tile) {
+    const int units = batches * num_tiles;  // one unit = the `heads` workgroups of a (batch, tile)
+    int unit, head;
+    if ((units & 7) == 0) {
+        const int xcd = bid & 7, slot = bid >> 3;
+        unit = (slot / heads) * 8 + xcd;
+        head = slot % heads;
+    } else {
+        unit = bid / heads;
+        head = bid % heads;
+    }
+    *bh = (unit / num_tiles) * heads + head;
+    *tile = unit % num_tiles;
+}
+
+template <int MASK>
+__device__ __forceinline__ void map_block_for(const KParams& p, int bid, int num_tiles, int order, int* bh, int* tile) {
+    if (MASK != 0 && p.ms[1] == 0 && p.H > 1) map_block_shared_mask(bid, p.B, p.H, num_tiles, bh, tile);
+    else map_block(bid, p.B * p.H, num_tiles, order, bh, tile);
+}
+
+// ---------------------------------------------------------------- dropout bits shared inside a quad
+// A Philox call yields the 16 keep-bytes of a 4x4 block of P. In the MFMA register layouts the four
+// lanes of a quad (lanes 4n..4n+3) own four consecutive rows (forward, dQ) or four consecutive
+// columns (dK/dV) of the same blocks, so each of them would generate every block itself. Instead
+// lane q of the quad generates only the blocks of group q (mod 4) and the others fetch them with
+// quad-broadcast DPP moves: a quarter of the Philox work for 4 moves per block.
+template <int G>
+__device__ __forceinline__ uint32_t quad_bcast(uint32_t v) {
+    return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), G * 0x55, 0xf, 0xf, true));
+}
+// The block lane G of the quad holds, for every lane of the quad.
+template <int G>
+__device__ __forceinline__ Philox4 quad_bcast(const Philox4& r) {
+    Philox4 o;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) o.w[k] = quad_bcast<G>(r.w[k]);
+    return o;
+}
+// Same with the source lane as an argument (a constant once the caller's loop is unrolled).
+__device__ __forceinline__ Philox4 quad_bcast_from(int g, const Philox4& r) {
+    return g == 0 ? quad_bcast<0>(r) : (g == 1 ? quad_bcast<1>(r) : (g == 2 ? quad_bcast<2>(r) : quad_bcast<3>(r)));
+}
+// Row-owner form: this lane owns row i (i % 4 == lane % 4) and wants, for groups g = 0..3, the word
+// (4 key bytes) of keys key0 + gstride*g .. +3. `mine` is the block this lane generated for group
+// lane % 4, i.e. dropout_block(p, bh, i >> 2, (key0 + gstride * (lane % 4)) >> 2).
+__device__ __forceinline__ void quad_row_words(const Philox4& mine, int lane, uint32_t (&w)[4]) {
+    const int q = lane & 3;
+    const Philox4 b0 = quad_bcast<0>(mine), b1 = quad_bcast<1>(mine), b2 = quad_bcast<2>(mine), b3 = quad_bcast<3>(mine);
+    w[0] = q == 0 ? b0.w[0] : (q == 1 ? b0.w[1] : (q == 2 ? b0.w[2] : b0.w[3]));
+    w[1] = q == 0 ? b1.w[0] : (q == 1 ? b1.w[1] : (q == 2 ? b1.w[2] : b1.w[3]));
+    w[2] = q == 0 ? b2.w[0] : (q == 1 ? b2.w[1] : (q == 2 ? b2.w[2] : b2.w[3]));
+    w[3] = q == 0 ? b3.w[0] : (q == 1 ? b3.w[1] : (q == 2 ? b3.w[2] : b3.w[3]));
 }
 
 // Dropout bytes for 4 consecutive columns j0..j0+3 (j0 % 4 == 0) of row i: one 32-bit word.

@@ -44,7 +44,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     const bool stage_v = NW == 4 || wave < 4;      // which matrix this wave moves HBM -> LDS
     const bool stage_k = NW == 4 || wave >= 4;
     int bh, qt;
-    map_block(blockIdx.x, p.B * p.H, p.S / kBM, CAUSAL ? kHeavyLast : kUniformTiles, &bh, &qt);
+    map_block_for<MASK>(p, blockIdx.x, p.S / kBM, CAUSAL ? kHeavyLast : kUniformTiles, &bh, &qt);
     const int b = bh / p.H, hd = bh % p.H;
     const int q0 = qt * kBM;
     const int wrow0 = q0 + 32 * wave;  // first query row of this wave
@@ -219,14 +219,18 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
 #pragma unroll
                 for (int e = 0; e < 32; ++e) psum += x[e];
 #pragma unroll
-                for (int g = 0; g < 8; ++g) {
-                    const int key0 = t0 + 32 * (g >> 2) + 8 * (g & 3) + 4 * h;
-                    const uint32_t w = dropout_word(p, bh, qrow, key0);
+                for (int kb = 0; kb < 2; ++kb) {
+                    // group g of key block kb: keys t0 + 32 kb + 8 g + 4 h .. +3; this lane generates g = lane % 4
+                    const Philox4 mine = dropout_block(p, bh, qrow >> 2, (t0 + 32 * kb + 8 * (lane & 3) + 4 * h) >> 2);
+                    uint32_t w[4];
+                    quad_row_words(mine, lane, w);
 #pragma unroll
-                    for (int bb = 0; bb < 4; ++bb) {
-                        const bool keep = static_cast<int>((w >> (8 * bb)) & 0xffu) >= p.thr8;
-                        x[4 * g + bb] = keep ? x[4 * g + bb] * p.zscale : 0.f;
-                    }
+                    for (int g = 0; g < 4; ++g)
+#pragma unroll
+                        for (int bb = 0; bb < 4; ++bb) {
+                            const bool keep = static_cast<int>((w[g] >> (8 * bb)) & 0xffu) >= p.thr8;
+                            x[16 * kb + 4 * g + bb] = keep ? x[16 * kb + 4 * g + bb] * p.zscale : 0.f;
+                        }
                 }
             }
             // P as B operands; without dropout the row sum is taken from the rounded P that is
