@@ -34,7 +34,14 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     constexpr int DB = D / 32;  // 32-row blocks of O^T
     constexpr int kSteps = 2 * KK, kAhead = 8;
     constexpr int kPvSteps = 4 * DB, kPvAhead = 8;
-    __shared__ __attribute__((aligned(16))) char smem[kStages * kStageBytes];
+    // An fp32 mask block of a wave (32 rows x 64 keys) goes through a private 8 KiB LDS region when
+    // it fits (D = 64): lanes own rows, so direct loads would touch 32 cache lines per instruction,
+    // while LDS-direct loads fetch whole 256-byte rows and the swizzled tile is read back without
+    // bank conflicts. The region has the geometry of a 32-row SwzTile<128> (256-byte rows).
+    constexpr bool kMaskViaLds = MASK == kMaskF32 && D == 64;
+    using MaskTile = SwzTile<128>;
+    constexpr int kMaskBytes = 32 * MaskTile::kRowBytes;
+    __shared__ __attribute__((aligned(256))) char smem[kStages * kStageBytes + (kMaskViaLds ? NW * kMaskBytes : 0)];
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -68,6 +75,20 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     const int n_tiles = CAUSAL ? (q0 + kBM) / kBN : p.S / kBN;            // tiles the workgroup streams
     const int my_tiles = CAUSAL ? (wrow0 + 31) / kBN + 1 : n_tiles;       // tiles this wave has visible keys in
     const float c = p.scale_log2;
+
+    char* mask_lds = smem + kStages * kStageBytes + wave * kMaskBytes;
+    auto issue_mask = [&](int t) {  // mask block of tile t -> this wave's region (8 LDS-direct loads)
+        if constexpr (kMaskViaLds) {
+            const char* src = static_cast<const char*>(p.mask) +
+                              (b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(wrow0) * p.ms[2] + t * kBN) * 4;
+            int l = lane;
+            asm volatile("" : "+v"(l));  // offsets recomputed per tile rather than kept in registers
+#pragma unroll
+            for (int blk = 0; blk < kMaskBytes / 1024; ++blk)
+                lds_direct_load16(src, static_cast<uint32_t>(MaskTile::src_off(blk, l, p.ms[2] * 4)), mask_lds + blk * 1024);
+        }
+    };
+    issue_mask(0);
 
     // staging registers: with 8 waves a wave moves either K or V and one buffer serves both roles
     uint32_t sreg[StageRegs<D>::kCount];
@@ -122,7 +143,16 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
         float mk[MASK != kNoMask ? 32 : 1];
         if (active) {
             // additive mask for this lane's row: issued before the MFMAs, used after them
-            if constexpr (MASK != kNoMask) {
+            if constexpr (kMaskViaLds) {
+                // the block was requested a tile ago; nothing younger than it that is still needed in
+                // flight (the K/V registers of the next tile are stored right after the MFMAs)
+                TRI_WAIT_VMCNT(0);
+#pragma unroll
+                for (int g = 0; g < 8; ++g) {
+                    const f32x4 v = *reinterpret_cast<const f32x4*>(mask_lds + MaskTile::off(l32, 8 * (g >> 2) + 2 * (g & 3) + h));
+                    mk[4 * g + 0] = v.x; mk[4 * g + 1] = v.y; mk[4 * g + 2] = v.z; mk[4 * g + 3] = v.w;
+                }
+            } else if constexpr (MASK != kNoMask) {
                 const int64_t mrow = b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(qrow) * p.ms[2] + t0;
 #pragma unroll
                 for (int g = 0; g < 8; ++g) {
@@ -173,6 +203,15 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
             } else if (stage_v) {
                 TransStage<D>::store(sreg, nK + kKBytes, ltid);
                 if (j + 2 < n_tiles) TransStage<D>::load(sreg, vbase + (t0 + 2 * kBN) * vrow_bytes, vrow_bytes, ltid);
+            }
+        }
+
+        if constexpr (kMaskViaLds) {
+            // this tile's mask values are in registers: the region can take the next block. Issued after
+            // the staging block so that the compiler's wait for the staged registers does not cover it.
+            if (active && j + 1 < my_tiles) {
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                issue_mask(j + 1);
             }
         }
 

@@ -61,6 +61,7 @@ bool mfma_supported(int which, int dtype, const KParams& p) {
         if (p.mask_dtype != TRI_ATTN_F32 && p.mask_dtype != dtype) return false;
         if (!aligned16(p.mask)) return false;
         if ((p.ms[0] % 4) || (p.ms[1] % 4) || (p.ms[2] % 4)) return false;
+        if (p.ms[2] < 0 || p.ms[2] >= (int64_t{1} << 24)) return false;  // 32-bit offsets inside a mask block
     }
     switch (which) {
         case kMfmaFwd:
