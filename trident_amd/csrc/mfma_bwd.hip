@@ -44,7 +44,14 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
     constexpr int DB = D / 32;
     constexpr int kBlocksPerWave = 2 * Tile::kBlocks / NW;  // LDS-direct loads per wave and tile
     static_assert(2 * Tile::kBlocks % NW == 0, "tile blocks must divide among the waves");
-    __shared__ __attribute__((aligned(1024))) char smem[kStages * kStageBytes];
+    // An fp32 mask block of a wave (32 rows x 64 keys) goes through a private 8 KiB LDS region when
+    // it fits (D = 64): lanes own rows, so direct loads would touch 32 cache lines per instruction,
+    // while LDS-direct loads fetch whole 256-byte rows. Geometry of a 32-row SwzTile<128>.
+    constexpr bool kMaskViaLds = MASK == kMaskF32 && D == 64;
+    using MaskTile = SwzTile<128>;
+    constexpr int kMaskBytes = 32 * MaskTile::kRowBytes;
+    constexpr int kMaskLoads = kMaskBytes / 1024;
+    __shared__ __attribute__((aligned(1024))) char smem[kStages * kStageBytes + (kMaskViaLds ? NW * kMaskBytes : 0)];
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -105,6 +112,20 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
             lds_direct_load16(tile_src, src_off[i], stage + blk * 1024);
         }
     };
+    char* mask_lds = smem + kStages * kStageBytes + wave * kMaskBytes;
+    auto issue_mask = [&](int t) {  // mask block of tile t -> this wave's region
+        if constexpr (kMaskViaLds) {
+            const char* src = static_cast<const char*>(p.mask) +
+                              (b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(wrow0) * p.ms[2] + t * kBN) * 4;
+            int l = lane;
+            asm volatile("" : "+v"(l));  // offsets recomputed per tile rather than kept in registers
+#pragma unroll
+            for (int blk = 0; blk < kMaskLoads; ++blk)
+                lds_direct_load16(src, static_cast<uint32_t>(MaskTile::src_off(blk, l, p.ms[2] * 4)), mask_lds + blk * 1024);
+        }
+    };
+    // issue order: mask 0, tiles 0 1 2, then per tile j: mask j+1, tile j+3
+    issue_mask(0);
     issue_tile(0);
     if (1 < n_tiles) issue_tile(1);
     if (2 < n_tiles) issue_tile(2);
@@ -116,12 +137,25 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
         // tile j has landed (up to two younger tiles may still be in flight) and is visible to all
         // waves; every wave is done with tile j-1, whose slot takes the load of tile j+3
         {
-            const int younger = min(2, n_tiles - 1 - j);
+            // with a staged mask, block j must have landed too: only tile j+2 was issued after it
+            // (tiles 1 and 2 for j = 0)
+            const int younger = kMaskViaLds && j > 0 ? min(1, max(0, n_tiles - 2 - j)) : min(2, n_tiles - 1 - j);
             if (younger == 2) TRI_WAIT_VMCNT(2 * kBlocksPerWave);
             else if (younger == 1) TRI_WAIT_VMCNT(kBlocksPerWave);
             else TRI_WAIT_VMCNT(0);
         }
         lds_barrier();
+        float mk2[kMaskViaLds ? 32 : 1];
+        if constexpr (kMaskViaLds) {
+            // (a mask excludes the causal variant, so every wave works on every tile)
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                const f32x4 v = *reinterpret_cast<const f32x4*>(mask_lds + MaskTile::off(l32, 2 * g + h));
+                mk2[4 * g + 0] = v.x; mk2[4 * g + 1] = v.y; mk2[4 * g + 2] = v.z; mk2[4 * g + 3] = v.w;
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // region read before it is refilled
+            if (j + 1 < n_tiles) issue_mask(j + 1);
+        }
         if (j + 3 < n_tiles) issue_tile(j + 3);
         if (j >= my_tiles) continue;
 
@@ -132,7 +166,10 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
             float mk[MASK != kNoMask ? 16 : 1];
-            if constexpr (MASK != kNoMask) {
+            if constexpr (kMaskViaLds) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) mk[i] = mk2[16 * kb + i];
+            } else if constexpr (MASK != kNoMask) {
                 const int64_t mrow = b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(qrow) * p.ms[2] + t0 + 32 * kb;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) mk[i] = mask_at<T, MASK>(p.mask, mrow + c_row(i, h));
