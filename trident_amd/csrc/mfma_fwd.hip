@@ -2,12 +2,13 @@
 // D in {64,128}, S a multiple of 128 (replaces trident/kernel/attention.py:33-165).
 //
 // A workgroup of NW waves owns 32*NW query rows, one wave 32 of them. Q stays in registers as
-// the B operand of S^T = K Q^T; K (row-major, padded) and V^T (transposed, slot-permuted) tiles
-// of 64 keys live in a three-stage LDS ring that is filled through registers one tile ahead of
-// its use and loaded from HBM two tiles ahead. S^T and O^T = V^T P^T accumulate in fp32; P goes
-// from the S^T accumulators to the B operand of the second MFMA in registers. The row
-// statistics live one per lane; the two lane halves of a row are combined with one cross-lane
-// exchange per tile.
+// the B operand of S^T = K Q^T; K and V tiles of 64 keys live row-major (swizzled) in a four-stage
+// LDS ring filled by LDS-direct loads two tiles ahead: no staging registers, no address or
+// permute arithmetic on the vector ALU, whose issue slots the softmax needs. K is read as row
+// fragments, V^T through transposed LDS reads of the same row-major tile. S^T and O^T = V^T P^T
+// accumulate in fp32; P goes from the S^T accumulators to the B operand of the second MFMA in
+// registers. The row statistics live one per lane; the two lane halves of a row are combined
+// with one cross-lane exchange per tile.
 //
 // With 8 waves (two per SIMD) the upper four run one half-step behind the lower four: they
 // multiply the previous tile's P with V before they compute the scores of the current tile, so
@@ -19,17 +20,18 @@ namespace tri {
 namespace {
 
 constexpr int kBN = 64;      // keys per tile
-constexpr int kStages = 3;   // LDS ring depth
+constexpr int kStages = 4;   // LDS ring depth
 constexpr float kTau = 8.f;  // lazy-rescale threshold, log2 domain
 
 enum MaskKind { kNoMask = 0, kMaskF32 = 1, kMaskT = 2 };
 
 template <typename T, int D, int NW, bool CAUSAL, int MASK, bool DROPOUT>
 __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
+    using Tile = SwzTile<D>;
     constexpr int kBM = 32 * NW;
-    constexpr int kKBytes = RowTile<D>::bytes(kBN);
-    constexpr int kVBytes = TransTile::bytes(D);
-    constexpr int kStageBytes = kKBytes + kVBytes;
+    constexpr int kKBytes = Tile::kBytes;
+    constexpr int kStageBytes = 2 * Tile::kBytes;  // K tile, V tile
+    constexpr int kBlocksPerWave = 2 * Tile::kBlocks / NW;  // LDS-direct loads per wave and tile
     constexpr int KK = D / 16;  // K-steps of S^T
     constexpr int DB = D / 32;  // 32-row blocks of O^T
     constexpr int kSteps = 2 * KK, kAhead = 8;
@@ -41,15 +43,12 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     constexpr bool kMaskViaLds = MASK == kMaskF32 && D == 64;
     using MaskTile = SwzTile<128>;
     constexpr int kMaskBytes = 32 * MaskTile::kRowBytes;
-    __shared__ __attribute__((aligned(256))) char smem[kStages * kStageBytes + (kMaskViaLds ? NW * kMaskBytes : 0)];
+    __shared__ __attribute__((aligned(1024))) char smem[kStages * kStageBytes + (kMaskViaLds ? NW * kMaskBytes : 0)];
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63, l32 = lane & 31, h = lane >> 5;
-    const int ltid = tid & 255;                    // index within the 256 threads that stage one matrix
     const bool skew = NW == 8 && wave >= 4;        // runs P V one tile late
-    const bool stage_v = NW == 4 || wave < 4;      // which matrix this wave moves HBM -> LDS
-    const bool stage_k = NW == 4 || wave >= 4;
     int bh, qt;
     map_block_for<MASK>(p, blockIdx.x, p.S / kBM, CAUSAL ? kHeavyLast : kUniformTiles, &bh, &qt);
     const int b = bh / p.H, hd = bh % p.H;
@@ -66,6 +65,8 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk)
         qf[kk] = *reinterpret_cast<const u32x4*>(qbase + qrow * p.qs[2] * 2 + (2 * kk + h) * 16);
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) settle(qf[kk]);
 
     f32x16 oacc[DB];
 #pragma unroll
@@ -90,24 +91,29 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     };
     issue_mask(0);
 
-    // staging registers: with 8 waves a wave moves either K or V and one buffer serves both roles
-    uint32_t sreg[StageRegs<D>::kCount];
-    uint32_t sreg2[NW == 4 ? StageRegs<D>::kCount : 1];
-    if (stage_k) {
-        RowStage<D>::load(sreg, kbase, krow_bytes, ltid);
-        RowStage<D>::store(sreg, smem, ltid);
-        if (n_tiles > 1) RowStage<D>::load(sreg, kbase + kBN * krow_bytes, krow_bytes, ltid);
-    }
-    if constexpr (NW == 4) {
-        TransStage<D>::load(sreg2, vbase, vrow_bytes, ltid);
-        TransStage<D>::store(sreg2, smem + kKBytes, ltid);
-        if (n_tiles > 1) TransStage<D>::load(sreg2, vbase + kBN * vrow_bytes, vrow_bytes, ltid);
-    } else if (stage_v) {
-        TransStage<D>::load(sreg, vbase, vrow_bytes, ltid);
-        TransStage<D>::store(sreg, smem + kKBytes, ltid);
-        if (n_tiles > 1) TransStage<D>::load(sreg, vbase + kBN * vrow_bytes, vrow_bytes, ltid);
-    }
-    __syncthreads();
+    auto issue_tile = [&](int t) {  // K and V rows of tile t -> ring slot t % kStages
+        char* stage = smem + (t % kStages) * kStageBytes;
+        int l = lane;
+        asm volatile("" : "+v"(l));  // offsets recomputed per tile rather than kept in registers
+#pragma unroll
+        for (int i = 0; i < kBlocksPerWave; ++i) {
+            const int blk = wave * kBlocksPerWave + i;  // 0 .. 2*kBlocks-1 over the K tile then the V tile
+            const bool is_v = blk >= Tile::kBlocks;
+            const char* tile_src = is_v ? vbase + static_cast<int64_t>(t) * kBN * vrow_bytes
+                                        : kbase + static_cast<int64_t>(t) * kBN * krow_bytes;
+            const uint32_t off = static_cast<uint32_t>(Tile::src_off(is_v ? blk - Tile::kBlocks : blk, l, is_v ? vrow_bytes : krow_bytes));
+            lds_direct_load16(tile_src, off, stage + blk * 1024);
+        }
+    };
+    issue_tile(0);
+    if (n_tiles > 1) issue_tile(1);
+
+    const int row_off0 = Tile::off(l32, h);
+    const int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
+    // fragment s of the S^T operand (key block s / KK, K-step s % KK) and of the O^T operand
+    // (K-step s / DB = 16 keys, column block s % DB)
+    auto k_frag = [&](const char* sK, int s) { return lds_read16(sK, (row_off0 ^ ((s % KK) << 5)) + 32 * (s / KK) * Tile::kRowBytes); };
+    auto v_frag = [&](const char* sV, int s) { return Tile::tr_frag(sV, tr_off0 ^ ((s % DB) << 6), tr_off1 ^ ((s % DB) << 6), s / DB); };
 
     u32x4 pb[4];  // P of the current tile as four B operands (kept across the step by skewed waves)
 #pragma unroll
@@ -115,6 +121,15 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
 
     const int n_iter = NW == 8 ? n_tiles + 1 : n_tiles;
     for (int j = 0; j < n_iter; ++j) {
+        // tile j has landed (tile j+1 may still be in flight) and is visible to all waves; every
+        // wave is done with tile j-2 (the skewed waves read V of tile j-1 in this step), whose slot
+        // takes the load of tile j+2
+        if (j < n_tiles) {
+            if (j + 1 < n_tiles) TRI_WAIT_VMCNT(kBlocksPerWave);
+            else TRI_WAIT_VMCNT(0);
+        }
+        lds_barrier();
+        if (j + 2 < n_tiles) issue_tile(j + 2);
         const char* sK = smem + (j % kStages) * kStageBytes;
         const char* sV = sK + kKBytes;
         const int t0 = j * kBN;
@@ -125,14 +140,14 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
             u32x4 vring[kPvAhead];
 #pragma unroll
             for (int s = 0; s < kPvAhead; ++s)
-                vring[s] = lds_read16(pV, TransTile::read_off(32 * (s % DB) + l32, s / DB, h));
+                vring[s] = v_frag(pV, s);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int s = 0; s < kPvSteps; ++s) {
                 oacc[s % DB] = Mma<T>::run(vring[s % kPvAhead], pb[s / DB], oacc[s % DB]);
                 if (s + kPvAhead < kPvSteps) {
                     const int n = s + kPvAhead;
-                    vring[s % kPvAhead] = lds_read16(pV, TransTile::read_off(32 * (n % DB) + l32, n / DB, h));
+                    vring[s % kPvAhead] = v_frag(pV, n);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -144,9 +159,9 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
         if (active) {
             // additive mask for this lane's row: issued before the MFMAs, used after them
             if constexpr (kMaskViaLds) {
-                // the block was requested a tile ago; nothing younger than it that is still needed in
-                // flight (the K/V registers of the next tile are stored right after the MFMAs)
-                TRI_WAIT_VMCNT(0);
+                // the block was requested a tile ago; only the loads of tile j+2 are younger
+                if (j + 2 < n_tiles) TRI_WAIT_VMCNT(kBlocksPerWave);
+                else TRI_WAIT_VMCNT(0);
 #pragma unroll
                 for (int g = 0; g < 8; ++g) {
                     const f32x4 v = *reinterpret_cast<const f32x4*>(mask_lds + MaskTile::off(l32, 8 * (g >> 2) + 2 * (g & 3) + h));
@@ -171,7 +186,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
             u32x4 ring[kAhead];
 #pragma unroll
             for (int s = 0; s < kAhead; ++s)
-                ring[s] = lds_read16(sK, RowTile<D>::off(32 * (s / KK) + l32, 2 * (s % KK) + h));
+                ring[s] = k_frag(sK, s);
             __builtin_amdgcn_sched_barrier(0);
             f32x16 st[2] = {zero16(), zero16()};
 #pragma unroll
@@ -179,7 +194,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
                 st[s / KK] = Mma<T>::run(ring[s % kAhead], qf[s % KK], st[s / KK]);
                 if (s + kAhead < kSteps) {
                     const int n = s + kAhead;
-                    ring[s % kAhead] = lds_read16(sK, RowTile<D>::off(32 * (n / KK) + l32, 2 * (n % KK) + h));
+                    ring[s % kAhead] = k_frag(sK, n);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -190,25 +205,8 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
             }
         }
 
-        // ---- staging: tile j+1 registers -> LDS, tile j+2 HBM -> registers (runs under the MFMAs)
-        if (j + 1 < n_tiles) {
-            char* nK = smem + ((j + 1) % kStages) * kStageBytes;
-            if (stage_k) {
-                RowStage<D>::store(sreg, nK, ltid);
-                if (j + 2 < n_tiles) RowStage<D>::load(sreg, kbase + (t0 + 2 * kBN) * krow_bytes, krow_bytes, ltid);
-            }
-            if constexpr (NW == 4) {
-                TransStage<D>::store(sreg2, nK + kKBytes, ltid);
-                if (j + 2 < n_tiles) TransStage<D>::load(sreg2, vbase + (t0 + 2 * kBN) * vrow_bytes, vrow_bytes, ltid);
-            } else if (stage_v) {
-                TransStage<D>::store(sreg, nK + kKBytes, ltid);
-                if (j + 2 < n_tiles) TransStage<D>::load(sreg, vbase + (t0 + 2 * kBN) * vrow_bytes, vrow_bytes, ltid);
-            }
-        }
-
         if constexpr (kMaskViaLds) {
-            // this tile's mask values are in registers: the region can take the next block. Issued after
-            // the staging block so that the compiler's wait for the staged registers does not cover it.
+            // this tile's mask values are in registers: the region can take the next block
             if (active && j + 1 < my_tiles) {
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 issue_mask(j + 1);
@@ -290,20 +288,19 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
                 u32x4 vring[kPvAhead];
 #pragma unroll
                 for (int s = 0; s < kPvAhead; ++s)
-                    vring[s] = lds_read16(sV, TransTile::read_off(32 * (s % DB) + l32, s / DB, h));
+                    vring[s] = v_frag(sV, s);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int s = 0; s < kPvSteps; ++s) {
                     oacc[s % DB] = Mma<T>::run(vring[s % kPvAhead], pb[s / DB], oacc[s % DB]);
                     if (s + kPvAhead < kPvSteps) {
                         const int n = s + kPvAhead;
-                        vring[s % kPvAhead] = lds_read16(sV, TransTile::read_off(32 * (n % DB) + l32, n / DB, h));
+                        vring[s % kPvAhead] = v_frag(sV, n);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
         }
-        __syncthreads();
     }
 
     l += xor32(l);
