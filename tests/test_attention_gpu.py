@@ -160,6 +160,29 @@ def test_broadcast_masks_and_their_gradient(dtype, mshape, device):
     _check(device, dtype, q, k, v, d_o, mask=mask, mask_grad=True, tag=f"bmask{mshape}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_key_padding_mask_row_broadcast(dtype, device):
+    """[B,1,1,S] additive mask (one row for all queries, row stride 0), as a key-padding mask is given."""
+    B, H, S, D = 2, 3, 256, 64
+    q, k, v, d_o = _gen((B, H, S, D), 33, dtype)
+    mask = torch.zeros(B, 1, 1, S)
+    mask[0, ..., 200:] = float("-inf")
+    mask[1, ..., 131:] = float("-inf")
+    mask += 0.25 * torch.randn(B, 1, 1, S, generator=torch.Generator().manual_seed(34))
+    _check(device, dtype, q, k, v, d_o, mask=mask, tag="key-padding")
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_fp32_mask_many_tiles(D, device):
+    """fp32 mask shared by the heads over 8 key tiles and 2 workgroups per head: the staged mask path (D=64)
+    refills its LDS region every tile; D=128 takes the direct loads."""
+    B, H, S = 2, 2, 512
+    q, k, v, d_o = _gen((B, H, S, D), 35, torch.bfloat16)
+    mask = torch.randn(B, 1, S, S, generator=torch.Generator().manual_seed(36))
+    mask[..., 300:420] = float("-inf")
+    _check(device, torch.bfloat16, q, k, v, d_o, mask=mask, tag=f"fp32 mask D={D}")
+
+
 def test_mask_with_fully_masked_leading_tiles(device):
     """Keys [0, 192) masked for every row: the running max stays -inf over whole tiles."""
     B, H, S, D = 1, 2, 256, 64
