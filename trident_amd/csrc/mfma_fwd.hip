@@ -10,9 +10,9 @@
 // registers. The row statistics live one per lane; the two lane halves of a row are combined
 // with one cross-lane exchange per tile.
 //
-// With 8 waves (two per SIMD) the upper four run one half-step behind the lower four: they
-// multiply the previous tile's P with V before they compute the scores of the current tile, so
-// while one wave of a SIMD is in its softmax (vector ALU) the other one feeds the matrix pipe.
+// With 8 waves there are two per SIMD. All of them run the same schedule: running the second wave
+// of a SIMD half a tile out of phase (its P V one tile late) was measured 7 % slower, in the kernel
+// and in a register-only model of its instruction mix alike.
 #include "launch.hpp"
 #include "mfma_common.hpp"
 
@@ -48,7 +48,6 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63, l32 = lane & 31, h = lane >> 5;
-    const bool skew = NW == 8 && wave >= 4;        // runs P V one tile late
     int bh, qt;
     map_block_for<MASK>(p, blockIdx.x, p.S / kBM, CAUSAL ? kHeavyLast : kUniformTiles, &bh, &qt);
     const int b = bh / p.H, hd = bh % p.H;
@@ -107,6 +106,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     };
     issue_tile(0);
     if (n_tiles > 1) issue_tile(1);
+    if (n_tiles > 2) issue_tile(2);
 
     const int row_off0 = Tile::off(l32, h);
     const int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
@@ -115,43 +115,20 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     auto k_frag = [&](const char* sK, int s) { return lds_read16(sK, (row_off0 ^ ((s % KK) << 5)) + 32 * (s / KK) * Tile::kRowBytes); };
     auto v_frag = [&](const char* sV, int s) { return Tile::tr_frag(sV, tr_off0 ^ ((s % DB) << 6), tr_off1 ^ ((s % DB) << 6), s / DB); };
 
-    u32x4 pb[4];  // P of the current tile as four B operands (kept across the step by skewed waves)
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) pb[ks] = u32x4{0, 0, 0, 0};
-
-    const int n_iter = NW == 8 ? n_tiles + 1 : n_tiles;
-    for (int j = 0; j < n_iter; ++j) {
-        // tile j has landed (tile j+1 may still be in flight) and is visible to all waves; every
-        // wave is done with tile j-2 (the skewed waves read V of tile j-1 in this step), whose slot
-        // takes the load of tile j+2
-        if (j < n_tiles) {
-            if (j + 1 < n_tiles) TRI_WAIT_VMCNT(kBlocksPerWave);
+    for (int j = 0; j < n_tiles; ++j) {
+        // tile j has landed (up to two younger tiles may still be in flight) and is visible to all
+        // waves; every wave is done with tile j-1, whose slot takes the load of tile j+3
+        {
+            const int younger = min(2, n_tiles - 1 - j);
+            if (younger == 2) TRI_WAIT_VMCNT(2 * kBlocksPerWave);
+            else if (younger == 1) TRI_WAIT_VMCNT(kBlocksPerWave);
             else TRI_WAIT_VMCNT(0);
         }
         lds_barrier();
-        if (j + 2 < n_tiles) issue_tile(j + 2);
+        if (j + 3 < n_tiles) issue_tile(j + 3);
         const char* sK = smem + (j % kStages) * kStageBytes;
         const char* sV = sK + kKBytes;
         const int t0 = j * kBN;
-
-        // ---- skewed waves: O^T += V^T P^T of the previous tile
-        if (skew && j >= 1 && j - 1 < my_tiles) {
-            const char* pV = smem + ((j - 1) % kStages) * kStageBytes + kKBytes;
-            u32x4 vring[kPvAhead];
-#pragma unroll
-            for (int s = 0; s < kPvAhead; ++s)
-                vring[s] = v_frag(pV, s);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int s = 0; s < kPvSteps; ++s) {
-                oacc[s % DB] = Mma<T>::run(vring[s % kPvAhead], pb[s / DB], oacc[s % DB]);
-                if (s + kPvAhead < kPvSteps) {
-                    const int n = s + kPvAhead;
-                    vring[s % kPvAhead] = v_frag(pV, n);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
 
         const bool active = j < my_tiles;
         float x[32];  // scores of this lane: x[16*kb + i] is key t0 + 32*kb + c_row(i,h)
@@ -159,9 +136,12 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
         if (active) {
             // additive mask for this lane's row: issued before the MFMAs, used after them
             if constexpr (kMaskViaLds) {
-                // the block was requested a tile ago; only the loads of tile j+2 are younger
-                if (j + 2 < n_tiles) TRI_WAIT_VMCNT(kBlocksPerWave);
-                else TRI_WAIT_VMCNT(0);
+                // the block was requested a tile ago; only the loads of tile j+3 are younger (block 0
+                // precedes every tile load, and tile 0 has landed)
+                if (j > 0) {
+                    if (j + 3 < n_tiles) TRI_WAIT_VMCNT(kBlocksPerWave);
+                    else TRI_WAIT_VMCNT(0);
+                }
 #pragma unroll
                 for (int g = 0; g < 8; ++g) {
                     const f32x4 v = *reinterpret_cast<const f32x4*>(mask_lds + MaskTile::off(l32, 8 * (g >> 2) + 2 * (g & 3) + h));
@@ -272,6 +252,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
             }
             // P as B operands; without dropout the row sum is taken from the rounded P that is
             // actually multiplied with V, two values per instruction
+            u32x4 pb[4];
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) {
                 pb[ks] = pack8<T>(&x[8 * ks]);
@@ -283,8 +264,8 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
                 }
             }
             l += psum;
-            // non-skewed waves: O^T += V^T P^T now
-            if (!skew) {
+            // O^T += V^T P^T
+            {
                 u32x4 vring[kPvAhead];
 #pragma unroll
                 for (int s = 0; s < kPvAhead; ++s)
