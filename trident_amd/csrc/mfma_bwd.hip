@@ -79,13 +79,6 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
     if (lse == -INFINITY) lse = INFINITY;  // fully masked row: every probability is 0
     const float dlt = p.delta[static_cast<int64_t>(bh) * p.S + qrow];
     const float c = p.scale_log2;
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-        settle(qf[kk]);
-        settle(gf[kk]);
-    }
-    settle(lse);
-    settle(dlt);
 
     f32x16 acc[DB];
 #pragma unroll
@@ -129,6 +122,14 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
     issue_tile(0);
     if (1 < n_tiles) issue_tile(1);
     if (2 < n_tiles) issue_tile(2);
+    // (the row fragments were requested before the tiles, so both latencies overlap)
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+        settle(qf[kk]);
+        settle(gf[kk]);
+    }
+    settle(lse);
+    settle(dlt);
 
     const int row_off0 = Tile::off(l32, h);
     const int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
@@ -281,11 +282,6 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
         kf[kk] = *reinterpret_cast<const u32x4*>(kbase + static_cast<int64_t>(key) * p.ks[2] * 2 + (2 * kk + h) * 16);
         vf[kk] = *reinterpret_cast<const u32x4*>(vbase + static_cast<int64_t>(key) * p.vs[2] * 2 + (2 * kk + h) * 16);
     }
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-        settle(kf[kk]);
-        settle(vf[kk]);
-    }
     const float c = p.scale_log2;
 
     f32x16 dk[DB], dv[DB];
@@ -324,6 +320,12 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
     issue_tile(t_begin);
     if (t_begin + 1 < n_tiles) issue_tile(t_begin + 1);
     if (t_begin + 2 < n_tiles) issue_tile(t_begin + 2);
+    // (the K and V fragments were requested before the tiles, so both latencies overlap)
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+        settle(kf[kk]);
+        settle(vf[kk]);
+    }
 
     const int row_off0 = Tile::off(l32, h);
     const int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
@@ -500,11 +502,6 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
         kf[kk] = *reinterpret_cast<const u32x4*>(kbase + static_cast<int64_t>(key) * p.ks[2] * 2 + (2 * kk + h) * 16);
         vf[kk] = *reinterpret_cast<const u32x4*>(vbase + static_cast<int64_t>(key) * p.vs[2] * 2 + (2 * kk + h) * 16);
     }
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-        settle(kf[kk]);
-        settle(vf[kk]);
-    }
     const float c = p.scale_log2;
 
     f32x16 dk[DH], dv[DH];
@@ -541,6 +538,12 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
     };
     issue_tile(t_begin);
     if (t_begin + 1 < n_tiles) issue_tile(t_begin + 1);
+    // (the K and V fragments were requested before the tiles, so both latencies overlap)
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+        settle(kf[kk]);
+        settle(vf[kk]);
+    }
 
     const int row_off0 = Tile::off(l32, h);
     const int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
@@ -728,21 +731,19 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
         }
     }
 
-    char* dkrow = static_cast<char*>(p.dk) + (b * p.dks[0] + hd * p.dks[1] + static_cast<int64_t>(key) * p.dks[2]) * 2;
-    char* dvrow = static_cast<char*>(p.dv) + (b * p.dvs[0] + hd * p.dvs[1] + static_cast<int64_t>(key) * p.dvs[2]) * 2;
-#pragma unroll
-    for (int d = 0; d < DH; ++d) {
-        const int db = DH * member + d;
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            u32x2 a, e;
-            a.x = Mma<T>::pack2(dk[d][4 * g + 0] * p.scale, dk[d][4 * g + 1] * p.scale);
-            a.y = Mma<T>::pack2(dk[d][4 * g + 2] * p.scale, dk[d][4 * g + 3] * p.scale);
-            e.x = Mma<T>::pack2(dv[d][4 * g + 0], dv[d][4 * g + 1]);
-            e.y = Mma<T>::pack2(dv[d][4 * g + 2], dv[d][4 * g + 3]);
-            *reinterpret_cast<u32x2*>(dkrow + (32 * db + 8 * g + 4 * h) * 2) = a;
-            *reinterpret_cast<u32x2*>(dvrow + (32 * db + 8 * g + 4 * h) * 2) = e;
-        }
+    // every wave is out of the loop: the ring can serve as the waves' private transposition patches
+    lds_barrier();
+    {
+        using Store = RowBlockStore<T, DH>;
+        static_assert(NW * Store::kPatchBytes <= kStages * kStageBytes, "patches must fit into the ring");
+        char* patch = smem + wave * Store::kPatchBytes;
+        const int64_t row = wkey0;  // first key of this pair; this member writes columns 32*DH*member ..
+        char* dk0 = static_cast<char*>(p.dk) + (b * p.dks[0] + hd * p.dks[1] + row * p.dks[2] + 32 * DH * member) * 2;
+        char* dv0 = static_cast<char*>(p.dv) + (b * p.dvs[0] + hd * p.dvs[1] + row * p.dvs[2] + 32 * DH * member) * 2;
+        const float sc = p.scale;
+        Store::run(dk, [sc](float x) { return x * sc; }, patch, dk0, p.dks[2] * 2, lane);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // patch read before it is rewritten
+        Store::run(dv, [](float x) { return x; }, patch, dv0, p.dvs[2] * 2, lane);
     }
 }
 

@@ -369,6 +369,45 @@ __device__ __forceinline__ void map_block_for(const KParams& p, int bid, int num
     else map_block(bid, p.B * p.H, num_tiles, order, bh, tile);
 }
 
+// ---------------------------------------------------------------- coalesced epilogue
+// A wave holds NB transposed C tiles: lane = output row (l32, two lanes per row), 16 registers per
+// tile = 4 groups of 4 consecutive columns. Stored straight from registers, every store instruction
+// would touch 32 rows with 16 bytes each. Instead the wave writes its 32 x (32 NB) block of 16-bit
+// values into a private LDS patch (row pitch padded by 16 bytes) and reads it back with 16 bytes per
+// lane along the rows, so that a store instruction writes whole 64 NB-byte row segments.
+// `patch` must be private to the wave and no longer in use by anyone (barrier before the call).
+// `scale(i)` is applied per register; `row0` points at column 0 of the wave's first row.
+template <typename T, int NB>
+struct RowBlockStore {
+    static constexpr int kRowBytes = 64 * NB;
+    static constexpr int kPitch = kRowBytes + 16;
+    static constexpr int kPatchBytes = 32 * kPitch;
+    static constexpr int kLanesPerRow = kRowBytes / 16;
+    static constexpr int kRowsPerStore = 64 / kLanesPerRow;
+    template <typename Scale>
+    static __device__ __forceinline__ void run(const f32x16 (&acc)[NB], Scale scale, char* patch, char* row0,
+                                               int64_t row_stride_bytes, int lane) {
+        const int l32 = lane & 31, h = lane >> 5;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                u32x2 v;
+                v.x = Mma<T>::pack2(scale(acc[nb][4 * g + 0]), scale(acc[nb][4 * g + 1]));
+                v.y = Mma<T>::pack2(scale(acc[nb][4 * g + 2]), scale(acc[nb][4 * g + 3]));
+                lds_write8(patch, l32 * kPitch + (32 * nb + 8 * g + 4 * h) * 2, v);
+            }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // same wave wrote, same wave reads
+        const int r = lane / kLanesPerRow, c = lane % kLanesPerRow;
+#pragma unroll
+        for (int i = 0; i < 32 / kRowsPerStore; ++i) {
+            const int row = i * kRowsPerStore + r;
+            const u32x4 v = lds_read16(patch, row * kPitch + c * 16);
+            *reinterpret_cast<u32x4*>(row0 + row * row_stride_bytes + c * 16) = v;
+        }
+    }
+};
+
 // ---------------------------------------------------------------- dropout bits shared inside a quad
 // A Philox call yields the 16 keep-bytes of a 4x4 block of P. In the MFMA register layouts the four
 // lanes of a quad (lanes 4n..4n+3) own four consecutive rows (forward, dQ) or four consecutive

@@ -34,8 +34,8 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     constexpr int kBlocksPerWave = 2 * Tile::kBlocks / NW;  // LDS-direct loads per wave and tile
     constexpr int KK = D / 16;  // K-steps of S^T
     constexpr int DB = D / 32;  // 32-row blocks of O^T
-    constexpr int kSteps = 2 * KK, kAhead = 8;
-    constexpr int kPvSteps = 4 * DB, kPvAhead = 8;
+    constexpr int kSteps = 2 * KK, kAhead = 4;
+    constexpr int kPvSteps = 4 * DB, kPvAhead = 4;
     // An fp32 mask block of a wave (32 rows x 64 keys) goes through a private 8 KiB LDS region when
     // it fits (D = 64): lanes own rows, so direct loads would touch 32 cache lines per instruction,
     // while LDS-direct loads fetch whole 256-byte rows and the swizzled tile is read back without
@@ -64,8 +64,6 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk)
         qf[kk] = *reinterpret_cast<const u32x4*>(qbase + qrow * p.qs[2] * 2 + (2 * kk + h) * 16);
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) settle(qf[kk]);
 
     f32x16 oacc[DB];
 #pragma unroll
@@ -107,6 +105,9 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     issue_tile(0);
     if (n_tiles > 1) issue_tile(1);
     if (n_tiles > 2) issue_tile(2);
+    // (the Q fragments were requested before the tiles, so both latencies overlap)
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) settle(qf[kk]);
 
     const int row_off0 = Tile::off(l32, h);
     const int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
