@@ -226,16 +226,15 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
         }
     }
 
-    char* out = static_cast<char*>(p.dq) + (b * p.dqs[0] + hd * p.dqs[1] + static_cast<int64_t>(qrow) * p.dqs[2]) * 2;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            u32x2 v;
-            v.x = Mma<T>::pack2(acc[db][4 * g + 0] * p.scale, acc[db][4 * g + 1] * p.scale);
-            v.y = Mma<T>::pack2(acc[db][4 * g + 2] * p.scale, acc[db][4 * g + 3] * p.scale);
-            *reinterpret_cast<u32x2*>(out + (32 * db + 8 * g + 4 * h) * 2) = v;
-        }
+    // every wave is out of the loop: the ring can serve as the waves' private transposition patches
+    lds_barrier();
+    {
+        using Store = RowBlockStore<T, DB>;
+        static_assert(NW * Store::kPatchBytes <= kStages * kStageBytes, "patches must fit into the ring");
+        char* out0 = static_cast<char*>(p.dq) + (b * p.dqs[0] + hd * p.dqs[1] + static_cast<int64_t>(wrow0) * p.dqs[2]) * 2;
+        const float sc = p.scale;
+        Store::run(acc, [sc](float x) { return x * sc; }, smem + wave * Store::kPatchBytes, out0, p.dqs[2] * 2, lane);
+    }
 }
 
 // ------------------------------------------------------------------ dK, dV (8 waves)
@@ -435,20 +434,19 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
         }
     }
 
-    char* dkrow = static_cast<char*>(p.dk) + (b * p.dks[0] + hd * p.dks[1] + static_cast<int64_t>(key) * p.dks[2]) * 2;
-    char* dvrow = static_cast<char*>(p.dv) + (b * p.dvs[0] + hd * p.dvs[1] + static_cast<int64_t>(key) * p.dvs[2]) * 2;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            u32x2 a, e;
-            a.x = Mma<T>::pack2(dk[db][4 * g + 0] * p.scale, dk[db][4 * g + 1] * p.scale);
-            a.y = Mma<T>::pack2(dk[db][4 * g + 2] * p.scale, dk[db][4 * g + 3] * p.scale);
-            e.x = Mma<T>::pack2(dv[db][4 * g + 0], dv[db][4 * g + 1]);
-            e.y = Mma<T>::pack2(dv[db][4 * g + 2], dv[db][4 * g + 3]);
-            *reinterpret_cast<u32x2*>(dkrow + (32 * db + 8 * g + 4 * h) * 2) = a;
-            *reinterpret_cast<u32x2*>(dvrow + (32 * db + 8 * g + 4 * h) * 2) = e;
-        }
+    // every wave is out of the loop: the ring can serve as the waves' private transposition patches
+    lds_barrier();
+    {
+        using Store = RowBlockStore<T, DB>;
+        static_assert(NW * Store::kPatchBytes <= kStages * kStageBytes, "patches must fit into the ring");
+        char* patch = smem + wave * Store::kPatchBytes;
+        char* dk0 = static_cast<char*>(p.dk) + (b * p.dks[0] + hd * p.dks[1] + static_cast<int64_t>(wkey0) * p.dks[2]) * 2;
+        char* dv0 = static_cast<char*>(p.dv) + (b * p.dvs[0] + hd * p.dvs[1] + static_cast<int64_t>(wkey0) * p.dvs[2]) * 2;
+        const float sc = p.scale;
+        Store::run(dk, [sc](float x) { return x * sc; }, patch, dk0, p.dks[2] * 2, lane);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // patch read before it is rewritten
+        Store::run(dv, [](float x) { return x; }, patch, dv0, p.dvs[2] * 2, lane);
+    }
 }
 
 // ------------------------------------------------------------------ dK, dV (paired waves)

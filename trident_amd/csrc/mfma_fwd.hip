@@ -287,16 +287,14 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
 
     l += xor32(l);
     const float inv = 1.f / l;
-    char* orow = static_cast<char*>(p.o) + (b * p.os[0] + hd * p.os[1] + static_cast<int64_t>(qrow) * p.os[2]) * 2;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            u32x2 v;
-            v.x = Mma<T>::pack2(oacc[db][4 * g + 0] * inv, oacc[db][4 * g + 1] * inv);
-            v.y = Mma<T>::pack2(oacc[db][4 * g + 2] * inv, oacc[db][4 * g + 3] * inv);
-            *reinterpret_cast<u32x2*>(orow + (32 * db + 8 * g + 4 * h) * 2) = v;
-        }
+    // every wave is out of the loop: the ring can serve as the waves' private transposition patches
+    lds_barrier();
+    {
+        using Store = RowBlockStore<T, DB>;
+        static_assert(NW * Store::kPatchBytes <= kStages * kStageBytes, "patches must fit into the ring");
+        char* o0 = static_cast<char*>(p.o) + (b * p.os[0] + hd * p.os[1] + static_cast<int64_t>(wrow0) * p.os[2]) * 2;
+        Store::run(oacc, [inv](float x) { return x * inv; }, smem + wave * Store::kPatchBytes, o0, p.os[2] * 2, lane);
+    }
     if (h == 0) p.lse[static_cast<int64_t>(bh) * p.S + qrow] = m + fast_log2(l);
 }
 
