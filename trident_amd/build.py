@@ -22,6 +22,7 @@ FLAGS = [
     "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    "-Wno-inline-asm",  # the LDS-direct load helpers name M0 as clobbered, which clang reports as a reserved register
     "-I", INCLUDE,
     "-I", CSRC,
 ]
