@@ -10,8 +10,8 @@
 // delta are per-lane scalars, and a C tile can be fed back as the B operand of the next
 // MFMA without leaving registers: registers 8g .. 8g+7 of a C tile, converted to 16 bit,
 // are the 8 K-slots of K-step g; slot t of lane-half h then stands for tile row
-// 16g + 8*(t/4) + 4h + t%4, and the A operand of that MFMA is stored in LDS in exactly
-// that slot order ("slot-permuted" transposed tiles below).
+// 16g + 8*(t/4) + 4h + t%4, and the A operand of that MFMA must present its K dimension in
+// exactly that slot order, which is what the transposed LDS reads of SwzTile below deliver.
 #pragma once
 #include "common.hpp"
 
@@ -91,41 +91,10 @@ __device__ __forceinline__ int c_row(int i, int h) { return 8 * (i >> 2) + 4 * h
 
 __device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32); }
 
-// ---------------------------------------------------------------- LDS tiles
-// Row-major tile [ROWS][D] of 16-bit elements, rows padded by 16 bytes so that the 32 lanes
-// of an A-operand read (32 consecutive rows, same 16-byte column chunk) hit distinct banks.
-template <int D>
-struct RowTile {
-    static constexpr int kStride = D * 2 + 16;  // bytes
-    static constexpr int bytes(int rows) { return rows * kStride; }
-    // 16-byte chunk c of row r
-    static __device__ __forceinline__ int off(int r, int c) { return r * kStride + c * 16; }
-};
-
-// Transposed, slot-permuted tile of a [64][D] source: LDS row d (128 bytes) holds the 64
-// source rows of column d; source row r sits at slot 16*(r/16) + 8*((r/4)%2) + 4*((r/8)%2) + r%4,
-// and 16-byte chunks are XOR-swizzled with (d%8)^((d/8)%8) so that both the 8-byte writes
-// (16 lanes = 16 different d, stride 8) and the 16-byte A-operand reads (32 consecutive d) are
-// bank-conflict free.
-struct TransTile {
-    static constexpr int kRowBytes = 128;
-    static constexpr int bytes(int d) { return d * kRowBytes; }
-    static __device__ __forceinline__ int swz(int d) { return (d & 7) ^ ((d >> 3) & 7); }
-    // A operand: LDS row d, K-step ks (16 source rows), lane-half h
-    static __device__ __forceinline__ int read_off(int d, int ks, int h) {
-        return d * kRowBytes + (((2 * ks + h) ^ swz(d)) << 4);
-    }
-    // 8-byte write of source rows 4*rq .. 4*rq+3 (rq = 0..15) of column d
-    static __device__ __forceinline__ int write_off(int d, int rq) {
-        const int chunk = 2 * (rq >> 2) + (rq & 1);
-        return d * kRowBytes + ((chunk ^ swz(d)) << 4) + ((rq >> 1) & 1) * 8;
-    }
-};
-
+// ---------------------------------------------------------------- LDS access
 __device__ __forceinline__ u32x4 lds_read16(const char* smem, int off) {
     return *reinterpret_cast<const u32x4*>(smem + off);
 }
-__device__ __forceinline__ void lds_write16(char* smem, int off, u32x4 v) { *reinterpret_cast<u32x4*>(smem + off) = v; }
 __device__ __forceinline__ void lds_write8(char* smem, int off, u32x2 v) { *reinterpret_cast<u32x2*>(smem + off) = v; }
 
 // ---------------------------------------------------------------- swizzled tiles filled by LDS-direct loads
@@ -140,8 +109,6 @@ __device__ __forceinline__ void lds_write8(char* smem, int off, u32x2 v) { *rein
 //                  when lane j points at row (base + j/4), columns 4*(j%4) .. +3.
 // The transposed form yields the K-slot order of the C registers (see the top of this file)
 // without any permuted storage.
-#define TRI_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
-#define TRI_GLB_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
 // LDS-direct loads and the matching barrier, issued through inline assembly. The compiler's own
@@ -213,105 +180,6 @@ struct SwzTile {
 
 // s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14)
 #define TRI_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
-
-// ---------------------------------------------------------------- HBM -> registers -> LDS staging
-// One [64][D] tile of 16-bit elements is moved by 256 threads, D/8 registers each. Both layouts
-// below work on the same raw register array, so a wave that stages K and a wave that stages V
-// can share one buffer in code that serves both roles.
-template <int D>
-struct StageRegs {
-    static constexpr int kCount = D / 8;  // 16 for D=128, 8 for D=64
-};
-
-// Row-major target (RowTile<D>): thread t holds 16-byte chunks t, t+256, ... of the tile.
-template <int D>
-struct RowStage {
-    static constexpr int kChunksPerRow = D / 8;
-    static constexpr int kPerThread = 64 * kChunksPerRow / 256;  // 4 for D=128, 2 for D=64
-    static __device__ __forceinline__ void load(uint32_t (&r)[StageRegs<D>::kCount], const char* base,
-                                                int64_t row_stride_bytes, int tid) {
-#pragma unroll
-        for (int i = 0; i < kPerThread; ++i) {
-            const int g = tid + 256 * i;
-            const int row = g / kChunksPerRow, c = g % kChunksPerRow;
-            const u32x4 v = *reinterpret_cast<const u32x4*>(base + row * row_stride_bytes + c * 16);
-            r[4 * i + 0] = v.x; r[4 * i + 1] = v.y; r[4 * i + 2] = v.z; r[4 * i + 3] = v.w;
-        }
-    }
-    static __device__ __forceinline__ void store(const uint32_t (&r)[StageRegs<D>::kCount], char* smem, int tid) {
-#pragma unroll
-        for (int i = 0; i < kPerThread; ++i) {
-            const int g = tid + 256 * i;
-            const int row = g / kChunksPerRow, c = g % kChunksPerRow;
-            u32x4 v;
-            v.x = r[4 * i + 0]; v.y = r[4 * i + 1]; v.z = r[4 * i + 2]; v.w = r[4 * i + 3];
-            lds_write16(smem, RowTile<D>::off(row, c), v);
-        }
-    }
-};
-
-// Transposed target (TransTile): thread (rq, c) holds source rows 4rq..4rq+3, columns
-// c*D/16 .. (c+1)*D/16-1 in registers [a*kWords + w]. Eight consecutive lanes cover half a source
-// row (one 128- or 64-byte segment of the global load); the 16 lanes that an 8-byte LDS write
-// handles per clock are 8 column chunks x 2 row quads whose slots differ in the 8-byte half, so
-// with the XOR swizzle they fall into 16 different bank pairs. The same registers can also be
-// written row-major (store_rows) when a kernel needs both forms of a tile.
-template <int D>
-struct TransStage {
-    static constexpr int kCols = D / 16;      // 8 for D=128 (16-byte loads), 4 for D=64 (8-byte loads)
-    static constexpr int kWords = kCols / 2;
-    static __device__ __forceinline__ int col_chunk(int tid) { return (tid & 7) | (((tid >> 4) & 1) << 3); }
-    static __device__ __forceinline__ int row_quad(int tid) {
-        const int rest = tid >> 5;
-        return ((rest >> 1) << 2) | (((tid >> 3) & 1) << 1) | (rest & 1);
-    }
-    static __device__ __forceinline__ void load(uint32_t (&r)[StageRegs<D>::kCount], const char* base,
-                                                int64_t row_stride_bytes, int tid) {
-        const int rq = row_quad(tid), c = col_chunk(tid);
-#pragma unroll
-        for (int a = 0; a < 4; ++a) {
-            const char* src = base + (4 * rq + a) * row_stride_bytes + c * kCols * 2;
-            if constexpr (kWords == 4) {
-                const u32x4 v = *reinterpret_cast<const u32x4*>(src);
-                r[4 * a + 0] = v.x; r[4 * a + 1] = v.y; r[4 * a + 2] = v.z; r[4 * a + 3] = v.w;
-            } else {
-                const u32x2 v = *reinterpret_cast<const u32x2*>(src);
-                r[2 * a + 0] = v.x; r[2 * a + 1] = v.y;
-            }
-        }
-    }
-    static __device__ __forceinline__ void store_rows(const uint32_t (&r)[StageRegs<D>::kCount], char* smem, int tid) {
-        const int rq = row_quad(tid), c = col_chunk(tid);
-#pragma unroll
-        for (int a = 0; a < 4; ++a) {
-            const int off = (4 * rq + a) * RowTile<D>::kStride + c * kCols * 2;
-            if constexpr (kWords == 4) {
-                u32x4 v;
-                v.x = r[4 * a + 0]; v.y = r[4 * a + 1]; v.z = r[4 * a + 2]; v.w = r[4 * a + 3];
-                lds_write16(smem, off, v);
-            } else {
-                u32x2 v;
-                v.x = r[2 * a + 0]; v.y = r[2 * a + 1];
-                lds_write8(smem, off, v);
-            }
-        }
-    }
-    static __device__ __forceinline__ void store(const uint32_t (&r)[StageRegs<D>::kCount], char* smem, int tid) {
-        const int rq = row_quad(tid), c = col_chunk(tid);
-#pragma unroll
-        for (int wd = 0; wd < kWords; ++wd) {
-            // even column: low halves of the four rows; odd column: high halves
-            u32x2 ev, od;
-            ev.x = __builtin_amdgcn_perm(r[1 * kWords + wd], r[0 * kWords + wd], 0x05040100u);
-            ev.y = __builtin_amdgcn_perm(r[3 * kWords + wd], r[2 * kWords + wd], 0x05040100u);
-            od.x = __builtin_amdgcn_perm(r[1 * kWords + wd], r[0 * kWords + wd], 0x07060302u);
-            od.y = __builtin_amdgcn_perm(r[3 * kWords + wd], r[2 * kWords + wd], 0x07060302u);
-            const int d = c * kCols + 2 * wd;
-            lds_write8(smem, TransTile::write_off(d, rq), ev);
-            lds_write8(smem, TransTile::write_off(d + 1, rq), od);
-        }
-    }
-};
 
 // Workgroup -> (head, tile) mapping. Workgroups are dealt round-robin to the 8 XCDs, each with
 // its own L2, so every XCD is given whole heads (head % 8 == XCD). With uniform tiles the XCD
@@ -440,13 +308,6 @@ __device__ __forceinline__ void quad_row_words(const Philox4& mine, int lane, ui
     w[1] = q == 0 ? b1.w[0] : (q == 1 ? b1.w[1] : (q == 2 ? b1.w[2] : b1.w[3]));
     w[2] = q == 0 ? b2.w[0] : (q == 1 ? b2.w[1] : (q == 2 ? b2.w[2] : b2.w[3]));
     w[3] = q == 0 ? b3.w[0] : (q == 1 ? b3.w[1] : (q == 2 ? b3.w[2] : b3.w[3]));
-}
-
-// Dropout bytes for 4 consecutive columns j0..j0+3 (j0 % 4 == 0) of row i: one 32-bit word.
-__device__ __forceinline__ uint32_t dropout_word(const KParams& p, uint32_t bh, uint32_t i, uint32_t j0) {
-    const Philox4 r = dropout_block(p, bh, i >> 2, j0 >> 2);
-    const uint32_t s = i & 3;
-    return s == 0 ? r.w[0] : (s == 1 ? r.w[1] : (s == 2 ? r.w[2] : r.w[3]));
 }
 
 }  // namespace tri
