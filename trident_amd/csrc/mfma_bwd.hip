@@ -253,7 +253,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
     constexpr int KK = D / 16;
     constexpr int DB = D / 32;
     constexpr int kBlocksPerWave = 2 * Tile::kBlocks / NW;
-    constexpr int kLoadsPerTile = kBlocksPerWave + 1;            // + lse or delta (upper bound per wave)
+    constexpr int kLoadsPerTile = kBlocksPerWave + 1;            // + lse or delta: exact for every wave
     static_assert(2 * Tile::kBlocks % NW == 0, "tile blocks must divide among the waves");
     __shared__ __attribute__((aligned(1024))) char smem[kStages * kStageBytes];
 
@@ -311,10 +311,11 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
             char* dst = stage + (is_g ? Tile::kBytes + (blk - Tile::kBlocks) * 1024 : blk * 1024);
             lds_direct_load16(tile_src, src_off[i], dst);
         }
-        if (wave == 0)
-            lds_direct_load4(lse_base + t * kBN, lane * 4, stage + 2 * Tile::kBytes);
-        if (wave == NW - 1)
-            lds_direct_load4(delta_base + t * kBN, lane * 4, stage + 2 * Tile::kBytes + kBN * 4);
+        // every wave issues exactly one more load, so that the vmcnt bookkeeping is the same in all of
+        // them: even waves fetch the 64 lse values, odd waves the 64 delta values (duplicates land
+        // on the same bytes)
+        if (wave & 1) lds_direct_load4(delta_base + t * kBN, lane * 4, stage + 2 * Tile::kBytes + kBN * 4);
+        else lds_direct_load4(lse_base + t * kBN, lane * 4, stage + 2 * Tile::kBytes);
     };
     issue_tile(t_begin);
     if (t_begin + 1 < n_tiles) issue_tile(t_begin + 1);
@@ -471,7 +472,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
     constexpr int DB = D / 32;
     constexpr int DH = DB / 2;                                   // column blocks a pair member accumulates
     constexpr int kBlocksPerWave = 2 * Tile::kBlocks / NW;
-    constexpr int kLoadsPerTile = kBlocksPerWave + 1;
+    constexpr int kLoadsPerTile = kBlocksPerWave + 1;            // + lse or delta: exact for every wave
     __shared__ __attribute__((aligned(1024))) char smem[kStages * kStageBytes + kXchBytes];
     char* xch = smem + kStages * kStageBytes;
 
@@ -494,12 +495,6 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
     const float* lse_base = p.lse + static_cast<int64_t>(bh) * p.S;
     const float* delta_base = p.delta + static_cast<int64_t>(bh) * p.S;
 
-    u32x4 kf[KK], vf[KK];
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-        kf[kk] = *reinterpret_cast<const u32x4*>(kbase + static_cast<int64_t>(key) * p.ks[2] * 2 + (2 * kk + h) * 16);
-        vf[kk] = *reinterpret_cast<const u32x4*>(vbase + static_cast<int64_t>(key) * p.vs[2] * 2 + (2 * kk + h) * 16);
-    }
     const float c = p.scale_log2;
 
     f32x16 dk[DH], dv[DH];
@@ -519,7 +514,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
     const int t_begin = CAUSAL ? k0 / kBN : 0;
     const int n_tiles = p.S / kBN;
     auto issue_tile = [&](int t) {
-        char* stage = smem + (t % kStages) * kStageBytes;
+        char* stage = smem + ((t - t_begin) % kStages) * kStageBytes;  // slots count from the first tile
 #pragma unroll
         for (int i = 0; i < kBlocksPerWave; ++i) {
             const int blk = wave * kBlocksPerWave + i;
@@ -529,22 +524,49 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
             char* dst = stage + (is_g ? Tile::kBytes + (blk - Tile::kBlocks) * 1024 : blk * 1024);
             lds_direct_load16(tile_src, src_off[i], dst);
         }
-        if (wave == 0)
-            lds_direct_load4(lse_base + t * kBN, lane * 4, stage + 2 * Tile::kBytes);
-        if (wave == NW - 1)
-            lds_direct_load4(delta_base + t * kBN, lane * 4, stage + 2 * Tile::kBytes + kBN * 4);
+        // every wave issues exactly one more load, so that the vmcnt bookkeeping is the same in all of
+        // them: even waves fetch the 64 lse values, odd waves the 64 delta values (duplicates land
+        // on the same bytes)
+        if (wave & 1) lds_direct_load4(delta_base + t * kBN, lane * 4, stage + 2 * Tile::kBytes + kBN * 4);
+        else lds_direct_load4(lse_base + t * kBN, lane * 4, stage + 2 * Tile::kBytes);
     };
+    // The K and V rows of the workgroup (128 keys = two 64-row tiles each) also arrive through LDS:
+    // lanes own keys, so loading the fragments straight into registers would touch 32 cache lines
+    // per instruction (measured: 4.5 us of a 95 us workgroup), while LDS-direct loads fetch whole rows.
+    // They land in the third ring slot plus the exchange slots, which nobody uses before the loop.
+    char* kv_lds = smem + 2 * kStageBytes;
+    static_assert(kStageBytes + kXchBytes >= 4 * Tile::kBytes, "K and V must fit behind the first two ring slots");
+    static_assert(4 * Tile::kBlocks % NW == 0, "K/V blocks must divide among the waves");
+    constexpr int kKvLoads = 4 * Tile::kBlocks / NW;
+    {
+        const int64_t krow_bytes = p.ks[2] * 2, vrow_bytes = p.vs[2] * 2;
+#pragma unroll
+        for (int i = 0; i < kKvLoads; ++i) {
+            const int blk = wave * kKvLoads + i;           // 0 .. 4*kBlocks-1: K tile 0, K tile 1, V tile 0, V tile 1
+            const int tile = blk / Tile::kBlocks, b16 = blk % Tile::kBlocks;
+            const bool is_v = tile >= 2;
+            const int64_t rb = is_v ? vrow_bytes : krow_bytes;
+            const char* src = (is_v ? vbase : kbase) + (k0 + 64 * (tile & 1)) * rb;
+            lds_direct_load16(src, static_cast<uint32_t>(Tile::src_off(b16, lane, rb)), kv_lds + blk * 1024);
+        }
+    }
     issue_tile(t_begin);
     if (t_begin + 1 < n_tiles) issue_tile(t_begin + 1);
-    // (the K and V fragments were requested before the tiles, so both latencies overlap)
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-        settle(kf[kk]);
-        settle(vf[kk]);
-    }
 
     const int row_off0 = Tile::off(l32, h);
     const int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
+    // K and V have landed (the Q/dO tiles issued after them may still be in flight)
+    if (t_begin + 1 < n_tiles) TRI_WAIT_VMCNT(2 * kLoadsPerTile);
+    else TRI_WAIT_VMCNT(kLoadsPerTile);
+    lds_barrier();
+    u32x4 kf[KK], vf[KK];
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+        const int off = (row_off0 ^ (kk << 5)) + 32 * (kb & 1) * Tile::kRowBytes;
+        kf[kk] = lds_read16(kv_lds + (kb >> 1) * Tile::kBytes, off);
+        vf[kk] = lds_read16(kv_lds + (2 + (kb >> 1)) * Tile::kBytes, off);
+    }
+    lds_barrier();  // every wave has its fragments: the region is free for the exchange slots and tile 2
     char* my_xch = xch + wave * 4096 + lane * 16;
     const char* peer_xch = xch + (wave ^ 4) * 4096 + lane * 16;
 
@@ -577,7 +599,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
         const int j = t_begin + lt;
         const int rb = j * kBN + 32 * member;
         if (lt < n_local && (!CAUSAL || rb + 31 >= wkey0)) {
-            const char* sQ = smem + (j % kStages) * kStageBytes;
+            const char* sQ = smem + (lt % kStages) * kStageBytes;
             const char* sG = sQ + Tile::kBytes;
             const float* sLse = reinterpret_cast<const float*>(sG + Tile::kBytes);
             const float* sDelta = sLse + kBN;
@@ -677,7 +699,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
         const int j = t_begin + lt;
         const int r0 = j * kBN;
         if (lt >= 0 && lt < n_local && (!CAUSAL || r0 + kBN - 1 >= wkey0)) {
-            const char* sQ = smem + (j % kStages) * kStageBytes;
+            const char* sQ = smem + (lt % kStages) * kStageBytes;
             const char* sG = sQ + Tile::kBytes;
             u32x4 pp[2], ps[2];  // the partner's P and dS
 #pragma unroll

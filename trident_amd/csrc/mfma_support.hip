@@ -68,7 +68,7 @@ bool mfma_supported(int which, int dtype, const KParams& p) {
             return aligned16(p.o) && strides8(p.os);
         case kMfmaDkdv:
             // the streamed tiles are addressed with 32-bit byte offsets from a per-tile base
-            if (!tile_offsets_fit(p.qs) || !tile_offsets_fit(p.dos)) return false;
+            if (!tile_offsets_fit(p.qs) || !tile_offsets_fit(p.dos) || !tile_offsets_fit(p.ks) || !tile_offsets_fit(p.vs)) return false;
             return aligned16(p.d_o) && strides8(p.dos) && aligned16(p.dk) && strides8(p.dks) && aligned16(p.dv) &&
                    strides8(p.dvs);
         case kMfmaDq:
