@@ -118,6 +118,39 @@ def run_steps(path, steps, warmup):
     return wall_ms, per_kernel
 
 
+def operator_ms(w, dev, steps, warmup):
+    """The same step through the operator API (trident_amd.function + autograd): what a user of the
+    reference's interface sees, including output allocation and the Python wrapper."""
+    import torch
+
+    import trident_amd
+    from trident_amd import workloads
+
+    q, k, v, d_o, mask = workloads.make_inputs(w)
+    q, k, v, d_o = [x.to(dev) for x in (q, k, v, d_o)]
+    mask = None if mask is None else mask.to(dev)
+    if w.dropout_p:
+        trident_amd.config.dropout_seed = (w.dropout_seed, 0)
+    for x in (q, k, v):
+        x.requires_grad_(w.backward)
+
+    def step():
+        out = trident_amd.function.scaled_dot_product_attention(q, k, v, attn_mask=mask, dropout_p=w.dropout_p,
+                                                                is_causal=w.is_causal)
+        if w.backward:
+            out.backward(d_o)
+            q.grad = k.grad = v.grad = None
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
 def cpu_baseline(w, reps=3):
     """torch.nn.functional.scaled_dot_product_attention on the host cores (the op the reference's
     tests take as their oracle), forward (+ backward) on the same workload."""
@@ -237,6 +270,9 @@ def main():
         gbs = nbytes / per_kernel["bwd_delta"] / 1e6
         result["delta_prepass"] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                    "frac": round(gbs / HBM_PEAK_GBS, 4)}
+    op_ms = operator_ms(w, dev, a.steps, a.warmup)
+    result["operator_api"] = {"ms_per_step": round(op_ms, 5), "tflops": round(flops_step / op_ms / 1e9, 1),
+                              "note": "same step through function.scaled_dot_product_attention + autograd"}
     if not a.no_cpu:
         result["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(result), flush=True)
