@@ -255,7 +255,14 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
     constexpr int kBlocksPerWave = 2 * Tile::kBlocks / NW;
     constexpr int kLoadsPerTile = kBlocksPerWave + 1;            // + lse or delta: exact for every wave
     static_assert(2 * Tile::kBlocks % NW == 0, "tile blocks must divide among the waves");
-    __shared__ __attribute__((aligned(1024))) char smem[kStages * kStageBytes];
+    // An fp32 mask block of a wave (64 rows x its 32 keys) goes through a private 8 KiB LDS region when
+    // it fits (D = 64). Plain loads would be tracked by the compiler, whose waits for them also drain
+    // the LDS-direct tile loads issued in between (the counter completes in order), which makes the
+    // tile prefetch synchronous. Geometry of a 64-row SwzTile<64> (128-byte rows = 32 keys).
+    constexpr bool kMaskViaLds = MASK == kMaskF32 && D == 64;
+    using MaskTile = SwzTile<64>;
+    constexpr int kMaskLoads = MaskTile::kBlocks;
+    __shared__ __attribute__((aligned(1024))) char smem[kStages * kStageBytes + (kMaskViaLds ? NW * MaskTile::kBytes : 0)];
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -317,6 +324,20 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
         if (wave & 1) lds_direct_load4(delta_base + t * kBN, lane * 4, stage + 2 * Tile::kBytes + kBN * 4);
         else lds_direct_load4(lse_base + t * kBN, lane * 4, stage + 2 * Tile::kBytes);
     };
+    char* mask_lds = smem + kStages * kStageBytes + wave * MaskTile::kBytes;
+    auto issue_mask = [&](int t) {  // rows of tile t x this wave's keys -> the wave's region
+        if constexpr (kMaskViaLds) {
+            const char* src = static_cast<const char*>(p.mask) +
+                              (b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(t) * kBN * p.ms[2] + wkey0) * 4;
+            int l = lane;
+            asm volatile("" : "+v"(l));  // offsets recomputed per tile rather than kept in registers
+#pragma unroll
+            for (int blk = 0; blk < kMaskLoads; ++blk)
+                lds_direct_load16(src, static_cast<uint32_t>(MaskTile::src_off(blk, l, p.ms[2] * 4)), mask_lds + blk * 1024);
+        }
+    };
+    // issue order: mask block of the first tile, three tiles, then per tile j: mask j+1, tile j+3
+    issue_mask(t_begin);
     issue_tile(t_begin);
     if (t_begin + 1 < n_tiles) issue_tile(t_begin + 1);
     if (t_begin + 2 < n_tiles) issue_tile(t_begin + 2);
@@ -332,12 +353,23 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
 
     for (int j = t_begin; j < n_tiles; ++j) {
         {
-            const int younger = min(2, n_tiles - 1 - j);
+            // with a staged mask, block j must have landed too: only tile j+2 was issued after it
+            // (two tiles after the first block)
+            const int younger = kMaskViaLds && j > t_begin ? min(1, max(0, n_tiles - 2 - j)) : min(2, n_tiles - 1 - j);
             if (younger == 2) TRI_WAIT_VMCNT(2 * kLoadsPerTile);
             else if (younger == 1) TRI_WAIT_VMCNT(kLoadsPerTile);
             else TRI_WAIT_VMCNT(0);
         }
         lds_barrier();
+        float mk2[kMaskViaLds ? 32 : 1];
+        if constexpr (kMaskViaLds) {
+            // (a mask excludes the causal variant, so every wave works on every tile)
+#pragma unroll
+            for (int i = 0; i < 32; ++i)
+                mk2[i] = *reinterpret_cast<const float*>(mask_lds + MaskTile::off(32 * (i >> 4) + c_row(i & 15, h), l32 >> 2) + (l32 & 3) * 4);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // region read before it is refilled
+            if (j + 1 < n_tiles) issue_mask(j + 1);
+        }
         if (j + 3 < n_tiles) issue_tile(j + 3);
         if (j < my_begin) continue;
 
@@ -352,7 +384,10 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
             const int rb = r0 + 32 * qb;
             if (CAUSAL && rb + 31 < wkey0) continue;  // whole block above the wave's keys
             float mk[MASK != kNoMask ? 16 : 1];
-            if constexpr (MASK != kNoMask) {
+            if constexpr (kMaskViaLds) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) mk[i] = qb ? mk2[16 + i] : mk2[i];  // static indices keep it in registers
+            } else if constexpr (MASK != kNoMask) {
                 const int64_t mbase = b * p.ms[0] + hd * p.ms[1] + key;
 #pragma unroll
                 for (int i = 0; i < 16; ++i)
