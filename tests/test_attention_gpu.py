@@ -251,6 +251,52 @@ def test_dropout_extremes_and_determinism(device):
     assert torch.equal(a, b) and not torch.equal(a, c)
 
 
+# ------------------------------------------------------------------ lengths the operator API rejects
+def _abi_case(device, dtype, S, D, variant, seed):
+    """The operator API accepts power-of-two lengths only (reference rule); the C ABI takes any
+    length.  This calls the ABI wrappers directly: a multiple of 128 that is not one of 256 runs the
+    4-wave matrix-core kernels over several tiles, other lengths run the general kernels."""
+    from trident_amd.operation import Attention
+    q, k, v, d_o = _gen((1, 2, S, D), seed, dtype)
+    mask, causal, p = None, False, 0.0
+    if variant == "causal":
+        causal = True
+    elif variant == "mask":
+        mask = torch.randn(1, 2, S, S, generator=torch.Generator().manual_seed(seed + 1))
+    elif variant == "mask16":
+        mask = torch.randn(1, 1, S, S, generator=torch.Generator().manual_seed(seed + 1)).to(dtype)
+    elif variant == "causal+dropout":
+        causal, p = True, 0.2
+    scale = 1.0 / math.sqrt(D)
+    rng = (977, 3) if p > 0 else (0, 0)
+    tq, tk, tv, tdo = [x.to(device) for x in (q, k, v, d_o)]
+    tm = None if mask is None else mask.to(device)
+    o, lse = Attention._forward(tq, tk, tv, tm, p, causal, scale, *rng)
+    dq, dk, dv, _ = Attention._backward(tdo, tq, tk, tv, o, lse, tm, scale, p, causal, *rng, False)
+    kw = dict(mask=mask, dropout_p=p, is_causal=causal, scale=scale, seed=rng[0], offset=rng[1])
+    tag = f"abi S={S} D={D} {variant}"
+    o_ref, _ = parity.oracle_forward(q, k, v, **kw)
+    parity.close(o, o_ref, dtype, tag + " O")
+    dq_r, dk_r, dv_r, _, _ = parity.oracle_backward(q, k, v, d_o, o=o, **kw)
+    _, a_dq, a_dk, a_dv = parity.oracle_abs_sums(q, k, v, d_o, o=o, **kw)
+    parity.close(dq, dq_r, dtype, tag + " dQ", a_dq)
+    parity.close(dk, dk_r, dtype, tag + " dK", a_dk)
+    parity.close(dv, dv_r, dtype, tag + " dV", a_dv)
+
+
+@pytest.mark.parametrize("variant", ["plain", "causal", "mask", "mask16", "causal+dropout"])
+@pytest.mark.parametrize("S,D", [(384, 64), (384, 128), (640, 64), (640, 128)])
+def test_four_wave_kernels_over_several_tiles(S, D, variant, device):
+    _abi_case(device, torch.bfloat16, S, D, variant, 200 + S + D)
+
+
+@pytest.mark.parametrize("variant", ["plain", "causal", "mask", "causal+dropout"])
+@pytest.mark.parametrize("dtype,S,D", [(torch.float32, 100, 32), (torch.bfloat16, 200, 64), (torch.float16, 72, 128),
+                                       (torch.float32, 384, 64)])
+def test_lengths_that_are_not_powers_of_two(dtype, S, D, variant, device):
+    _abi_case(device, dtype, S, D, variant, 300 + S + D)
+
+
 # ------------------------------------------------------------------ full-size properties
 def test_config3_full_size_properties(device):
     """At B=2,H=16,S=4096,D=128 the oracle is too slow for the whole tensor; check it on a few
