@@ -90,6 +90,12 @@ __device__ __forceinline__ f32x16 zero16() {
 __device__ __forceinline__ int c_row(int i, int h) { return 8 * (i >> 2) + 4 * h + (i & 3); }
 
 __device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32); }
+// max / sum of a value with the one in lane ^ 32, exchanged on the vector ALU (no LDS round trip):
+// the swap leaves {x[l % 32], x[l % 32 + 32]} in the two registers of every lane. The instruction
+// needs two wait states after a vector write of its operands.
+__device__ __forceinline__ void swap32(float& a, float& b) { asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
+__device__ __forceinline__ float max_xor32(float x) { float a = x, b = x; swap32(a, b); return fmaxf(a, b); }
+__device__ __forceinline__ float sum_xor32(float x) { float a = x, b = x; swap32(a, b); return a + b; }
 
 // ---------------------------------------------------------------- LDS access
 __device__ __forceinline__ u32x4 lds_read16(const char* smem, int off) {

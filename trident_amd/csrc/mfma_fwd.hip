@@ -3,16 +3,24 @@
 //
 // A workgroup of NW waves owns 32*NW query rows, one wave 32 of them. Q stays in registers as
 // the B operand of S^T = K Q^T; K and V tiles of 64 keys live row-major (swizzled) in a four-stage
-// LDS ring filled by LDS-direct loads two tiles ahead: no staging registers, no address or
+// LDS ring filled by LDS-direct loads two or three tiles ahead: no staging registers, no address or
 // permute arithmetic on the vector ALU, whose issue slots the softmax needs. K is read as row
 // fragments, V^T through transposed LDS reads of the same row-major tile. S^T and O^T = V^T P^T
 // accumulate in fp32; P goes from the S^T accumulators to the B operand of the second MFMA in
 // registers. The row statistics live one per lane; the two lane halves of a row are combined
 // with one cross-lane exchange per tile.
 //
-// With 8 waves there are two per SIMD. All of them run the same schedule: running the second wave
-// of a SIMD half a tile out of phase (its P V one tile late) was measured 7 % slower, in the kernel
-// and in a register-only model of its instruction mix alike.
+// With 8 waves there are two per SIMD (waves w and w+4), and they run in opposite phases: a tile is
+// a softmax phase (vector ALU: maximum, exponentials, conversion, the loads of a later tile) and a
+// matrix phase (P V of this tile, then S^T of the next one), with a workgroup barrier after each;
+// waves 4-7 run one phase behind waves 0-3. The matrix pipe then always has a wave feeding it
+// while the other wave of the SIMD occupies the vector ALU, instead of both waves doing the same
+// thing at once (MFMA and vector instructions share the SIMD's issue port, and a dependent vector
+// instruction waits out the ALU latency unless the other wave fills the gap). The softmax
+// denominator is accumulated by the matrix pipe too (an all-ones A operand), and without dropout
+// half of the exponentials are taken in the matrix phase, between the MFMAs, to balance the two.
+#include <type_traits>
+
 #include "launch.hpp"
 #include "mfma_common.hpp"
 
@@ -34,8 +42,9 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     constexpr int kBlocksPerWave = 2 * Tile::kBlocks / NW;  // LDS-direct loads per wave and tile
     constexpr int KK = D / 16;  // K-steps of S^T
     constexpr int DB = D / 32;  // 32-row blocks of O^T
-    constexpr int kSteps = 2 * KK, kAhead = 4;
-    constexpr int kPvSteps = 4 * DB, kPvAhead = 4;
+    constexpr int kSteps = 2 * KK;    // MFMAs of S^T per tile
+    constexpr int kPvSteps = 4 * DB;  // MFMAs of O^T per tile
+    constexpr int kRing = 6;          // operand fragments in flight
     // An fp32 mask block of a wave (32 rows x 64 keys) goes through a private 8 KiB LDS region when
     // it fits (D = 64): lanes own rows, so direct loads would touch 32 cache lines per instruction,
     // while LDS-direct loads fetch whole 256-byte rows and the swizzled tile is read back without
@@ -88,113 +97,211 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     };
     issue_mask(0);
 
-    auto issue_tile = [&](int t) {  // K and V rows of tile t -> ring slot t % kStages
-        char* stage = smem + (t % kStages) * kStageBytes;
-        int l = lane;
-        asm volatile("" : "+v"(l));  // offsets recomputed per tile rather than kept in registers
-#pragma unroll
-        for (int i = 0; i < kBlocksPerWave; ++i) {
-            const int blk = wave * kBlocksPerWave + i;  // 0 .. 2*kBlocks-1 over the K tile then the V tile
-            const bool is_v = blk >= Tile::kBlocks;
-            const char* tile_src = is_v ? vbase + static_cast<int64_t>(t) * kBN * vrow_bytes
-                                        : kbase + static_cast<int64_t>(t) * kBN * krow_bytes;
-            const uint32_t off = static_cast<uint32_t>(Tile::src_off(is_v ? blk - Tile::kBlocks : blk, l, is_v ? vrow_bytes : krow_bytes));
-            lds_direct_load16(tile_src, off, stage + blk * 1024);
-        }
+    // A wave fetches blocks wave, wave + NW, ... of the K tile and of the V tile: their rows are a
+    // multiple of 16 apart, so one per-lane source offset (row within the block, swizzled chunk)
+    // serves all of them and the rest of the address is scalar arithmetic.
+    constexpr int kPerOperand = Tile::kBlocks / NW;
+    constexpr int kRowStep = NW * Tile::kRowsPerBlock;
+    static_assert(kRowStep % 16 == 0 && 2 * kPerOperand == kBlocksPerWave, "block assignment");
+    const uint32_t koff = static_cast<uint32_t>(Tile::src_off(wave, lane, krow_bytes));
+    const uint32_t voff = static_cast<uint32_t>(Tile::src_off(wave, lane, vrow_bytes));
+    // load number idx (0 .. kBlocksPerWave-1) of this wave's share of tile t -> ring slot t % kStages
+    auto issue_load = [&](int t, int idx) {
+        char* stage = smem + (t % kStages) * kStageBytes + wave * 1024;
+        const int i = idx % kPerOperand;
+        if (idx < kPerOperand)
+            lds_direct_load16(kbase + (static_cast<int64_t>(t) * kBN + i * kRowStep) * krow_bytes, koff, stage + i * NW * 1024);
+        else
+            lds_direct_load16(vbase + (static_cast<int64_t>(t) * kBN + i * kRowStep) * vrow_bytes, voff, stage + kKBytes + i * NW * 1024);
     };
+    // The loads of a tile are issued in four slices spread over the softmax phase: a wave stalls on a
+    // load until the memory pipeline accepts it, and sixteen loads arriving at once from the four
+    // waves of a group queue up for hundreds of cycles.
+    auto issue_slice = [&](int t, int part) {
+#pragma unroll
+        for (int idx = 0; idx < kBlocksPerWave; ++idx)
+            if (idx % 4 == part) issue_load(t, idx);
+    };
+    auto issue_tile = [&](int t) {
+#pragma unroll
+        for (int part = 0; part < 4; ++part) issue_slice(t, part);
+    };
+    // Ping-pong schedule (8 waves): waves w and w+4 share a SIMD. The loop alternates a softmax
+    // phase (vector ALU only) and a matrix phase (P V of this tile, then S^T of the next), with a
+    // barrier after each; the waves of group 1 run one phase behind those of group 0, so that a SIMD
+    // always has one wave issuing MFMAs and one issuing vector instructions instead of both doing
+    // the same thing at once. Group 0 may request tiles 2 ahead, group 1 (one phase later) 3 ahead.
+    constexpr bool kPingPong = NW == 8;
+    const int group = kPingPong ? wave >> 2 : 0;
+    const int dist = 2 + group;
+    auto wait_loads = [&](bool mask_block, bool tile) {  // all but the youngest (mask block, tile) have landed
+        constexpr int kM = kMaskBytes / 1024, kB = kBlocksPerWave;
+        if (mask_block && tile) TRI_WAIT_VMCNT(kM + kB);
+        else if (mask_block) TRI_WAIT_VMCNT(kM);
+        else if (tile) TRI_WAIT_VMCNT(kB);
+        else TRI_WAIT_VMCNT(0);
+    };
+    const int n_first = min(dist, n_tiles);
     issue_tile(0);
-    if (n_tiles > 1) issue_tile(1);
-    if (n_tiles > 2) issue_tile(2);
+    if (n_first > 1) issue_tile(1);
+    if (n_first > 2) issue_tile(2);
     // (the Q fragments were requested before the tiles, so both latencies overlap)
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) settle(qf[kk]);
 
-    const int row_off0 = Tile::off(l32, h);
-    const int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
+    int row_off0 = Tile::off(l32, h);
+    int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
     // fragment s of the S^T operand (key block s / KK, K-step s % KK) and of the O^T operand
     // (K-step s / DB = 16 keys, column block s % DB)
     auto k_frag = [&](const char* sK, int s) { return lds_read16(sK, (row_off0 ^ ((s % KK) << 5)) + 32 * (s / KK) * Tile::kRowBytes); };
     auto v_frag = [&](const char* sV, int s) { return Tile::tr_frag(sV, tr_off0 ^ ((s % DB) << 6), tr_off1 ^ ((s % DB) << 6), s / DB); };
 
-    for (int j = 0; j < n_tiles; ++j) {
-        // tile j has landed (up to two younger tiles may still be in flight) and is visible to all
-        // waves; every wave is done with tile j-1, whose slot takes the load of tile j+3
-        {
-            const int younger = min(2, n_tiles - 1 - j);
-            if (younger == 2) TRI_WAIT_VMCNT(2 * kBlocksPerWave);
-            else if (younger == 1) TRI_WAIT_VMCNT(kBlocksPerWave);
-            else TRI_WAIT_VMCNT(0);
-        }
-        lds_barrier();
-        if (j + 3 < n_tiles) issue_tile(j + 3);
-        const char* sK = smem + (j % kStages) * kStageBytes;
-        const char* sV = sK + kKBytes;
-        const int t0 = j * kBN;
+    f32x16 sc[2];  // scores of this lane: sc[kb][i] is key t0 + 32*kb + c_row(i,h)
+    float mk[MASK != kNoMask ? 32 : 1];
 
-        const bool active = j < my_tiles;
-        float x[32];  // scores of this lane: x[16*kb + i] is key t0 + 32*kb + c_row(i,h)
-        float mk[MASK != kNoMask ? 32 : 1];
-        if (active) {
-            // additive mask for this lane's row: issued before the MFMAs, used after them
-            if constexpr (kMaskViaLds) {
-                // the block was requested a tile ago; only the loads of tile j+3 are younger (block 0
-                // precedes every tile load, and tile 0 has landed)
-                if (j > 0) {
-                    if (j + 3 < n_tiles) TRI_WAIT_VMCNT(kBlocksPerWave);
-                    else TRI_WAIT_VMCNT(0);
-                }
+    // additive mask values of this lane's row for tile t, straight from memory
+    auto load_mask = [&](int t) {
+        if constexpr (MASK != kNoMask && !kMaskViaLds) {
+            const int64_t mrow = b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(qrow) * p.ms[2] + t * kBN;
 #pragma unroll
-                for (int g = 0; g < 8; ++g) {
-                    const f32x4 v = *reinterpret_cast<const f32x4*>(mask_lds + MaskTile::off(l32, 8 * (g >> 2) + 2 * (g & 3) + h));
+            for (int g = 0; g < 8; ++g) {
+                const int key0 = 32 * (g >> 2) + 8 * (g & 3) + 4 * h;
+                if constexpr (MASK == kMaskF32) {
+                    const f32x4 v = *reinterpret_cast<const f32x4*>(static_cast<const float*>(p.mask) + mrow + key0);
                     mk[4 * g + 0] = v.x; mk[4 * g + 1] = v.y; mk[4 * g + 2] = v.z; mk[4 * g + 3] = v.w;
-                }
-            } else if constexpr (MASK != kNoMask) {
-                const int64_t mrow = b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(qrow) * p.ms[2] + t0;
-#pragma unroll
-                for (int g = 0; g < 8; ++g) {
-                    const int key0 = 32 * (g >> 2) + 8 * (g & 3) + 4 * h;
-                    if constexpr (MASK == kMaskF32) {
-                        const f32x4 v = *reinterpret_cast<const f32x4*>(static_cast<const float*>(p.mask) + mrow + key0);
-                        mk[4 * g + 0] = v.x; mk[4 * g + 1] = v.y; mk[4 * g + 2] = v.z; mk[4 * g + 3] = v.w;
-                    } else {
-                        const u32x2 v = *reinterpret_cast<const u32x2*>(static_cast<const T*>(p.mask) + mrow + key0);
-                        mk[4 * g + 0] = Mma<T>::lo(v.x); mk[4 * g + 1] = Mma<T>::hi(v.x);
-                        mk[4 * g + 2] = Mma<T>::lo(v.y); mk[4 * g + 3] = Mma<T>::hi(v.y);
-                    }
+                } else {
+                    const u32x2 v = *reinterpret_cast<const u32x2*>(static_cast<const T*>(p.mask) + mrow + key0);
+                    mk[4 * g + 0] = Mma<T>::lo(v.x); mk[4 * g + 1] = Mma<T>::hi(v.x);
+                    mk[4 * g + 2] = Mma<T>::lo(v.y); mk[4 * g + 3] = Mma<T>::hi(v.y);
                 }
             }
-            // S^T = K Q^T with the A fragments requested kAhead MFMAs before their use
-            u32x4 ring[kAhead];
+        }
+    };
+    // mask block t from this wave's LDS region, then the request for block t+1
+    auto take_mask_block = [&](int t, bool first, bool tile_in_flight) {
+        if constexpr (kMaskViaLds) {
+            // block t was requested a matrix phase ago and only the newest tile load may be younger
+            // (block 0 precedes tile 0, which has landed)
+            if (!first) wait_loads(false, tile_in_flight);
 #pragma unroll
-            for (int s = 0; s < kAhead; ++s)
-                ring[s] = k_frag(sK, s);
+            for (int g = 0; g < 8; ++g) {
+                const f32x4 v = *reinterpret_cast<const f32x4*>(mask_lds + MaskTile::off(l32, 8 * (g >> 2) + 2 * (g & 3) + h));
+                mk[4 * g + 0] = v.x; mk[4 * g + 1] = v.y; mk[4 * g + 2] = v.z; mk[4 * g + 3] = v.w;
+            }
+            // the values are in registers: the region can take the next block
+            if (t + 1 < my_tiles) {
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                issue_mask(t + 1);
+            }
+        }
+    };
+    // The matrix phase of tile j: O^T += V^T P^T (steps 0 .. kPvSteps-1, skipped when WITH_PV is
+    // false) and then S^T = K Q^T of tile j+1 (when WITH_S). All A operands come through one ring of
+    // fragments requested kRing MFMAs before their use, across the boundary between the two products;
+    // the caller has requested the first kRing fragments.
+    u32x4 ring[kRing];
+    u32x4 pb[4];
+    // Without dropout the softmax denominator is accumulated by the matrix pipe as well: an all-ones
+    // A operand makes every row of the product the column sums of P^T, i.e. each lane holds (16
+    // times) the sum over ALL keys of its query row, taken from the same rounded P that multiplies
+    // V. With dropout the sum has to be taken before elements are dropped, on the vector ALU.
+    // Without dropout the exponentials of the second key block (and their conversion) are deferred into
+    // the matrix phase, one or two per MFMA of the first key block's P V steps: that phase has issue slots
+    // to spare, the softmax phase is the one the partner waits for.
+    constexpr bool kDefer = !DROPOUT;
+    float xd[16];        // deferred exponents (already scaled, masked) and then probabilities
+    float m_def = 0.f;   // the reference exponent they are taken against
+    const uint32_t one2 = Mma<T>::pack2(1.f, 1.f);
+    const u32x4 ones = {one2, one2, one2, one2};
+    f32x16 lacc = zero16();
+    auto frag = [&](auto with_pv, int j, int s) {
+        constexpr int pv = decltype(with_pv)::value ? kPvSteps : 0;
+        const char* stage_j = smem + ((j + kStages) % kStages) * kStageBytes;
+        const char* stage_n = smem + ((j + 1) % kStages) * kStageBytes;
+        return s < pv ? v_frag(stage_j + kKBytes, s) : k_frag(stage_n, s - pv);
+    };
+    auto matrix_phase = [&](auto with_pv, auto with_s, int j) {
+        constexpr int pv = decltype(with_pv)::value ? kPvSteps : 0;
+        constexpr int total = pv + (decltype(with_s)::value ? kSteps : 0);
+        if constexpr (decltype(with_s)::value) {
+            sc[0] = zero16();
+            sc[1] = zero16();
+        }
+#pragma unroll
+        for (int s = 0; s < total; ++s) {
+            if (s < pv) {
+                oacc[s % DB] = Mma<T>::run(ring[s % kRing], pb[s / DB], oacc[s % DB]);
+                // row sums of P (every accumulator row gets the same sum over the 16 keys)
+                if (!DROPOUT && s % DB == DB - 1) lacc = Mma<T>::run(ones, pb[s / DB], lacc);
+            } else {
+                const int s2 = s - pv;
+                sc[s2 / KK] = Mma<T>::run(ring[s % kRing], qf[s2 % KK], sc[s2 / KK]);
+            }
+            if (s + kRing < total) {
+                const int n = s + kRing;
+                ring[s % kRing] = frag(with_pv, j, n);
+            }
+            if constexpr (kDefer && pv > 0) {
+                // group 2 (B operand of K-step 2, first used at step 2 DB) during steps 0 .. 2 DB - 1,
+                // group 3 (first used at step 3 DB) during steps 2 DB .. 3 DB - 1
+                if (s < 3 * DB) {
+                    const int g = s < 2 * DB ? 2 : 3;
+                    const int w0 = g == 2 ? 0 : 2 * DB, n = g == 2 ? 2 * DB : DB;
+                    const int ne = n > 2 ? n - 2 : 1;           // steps that take exponentials
+                    const int pack_step = ne < n - 1 ? ne : n - 1;
+                    const int ls = s - w0;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (e * ne / 8 == ls) {
+                            float& v = xd[8 * (g - 2) + e];
+                            if constexpr (MASK == kNoMask) v = fast_exp2(fmaf(v, c, -m_def));
+                            else v = fast_exp2(v - m_def);
+                        }
+                    if (ls == pack_step) pb[g] = pack8<T>(&xd[8 * (g - 2)]);
+                }
+            }
             __builtin_amdgcn_sched_barrier(0);
-            f32x16 st[2] = {zero16(), zero16()};
+        }
+    };
+    using Yes = std::integral_constant<bool, true>;
+    using No = std::integral_constant<bool, false>;
+
+    // tile 0 has landed and is visible to all waves
+    if (n_first == 3) TRI_WAIT_VMCNT(2 * kBlocksPerWave);
+    else if (n_first == 2) TRI_WAIT_VMCNT(kBlocksPerWave);
+    else TRI_WAIT_VMCNT(0);
+    lds_barrier();
+    if (kPingPong && group == 1) {
+        // group 1 starts one phase late; group 0 reads tile 1 in its first matrix phase
+        if (n_first == 3) TRI_WAIT_VMCNT(kBlocksPerWave);
+        else TRI_WAIT_VMCNT(0);
+        lds_barrier();
+    }
+    {
+        load_mask(0);
 #pragma unroll
-            for (int s = 0; s < kSteps; ++s) {
-                st[s / KK] = Mma<T>::run(ring[s % kAhead], qf[s % KK], st[s / KK]);
-                if (s + kAhead < kSteps) {
-                    const int n = s + kAhead;
-                    ring[s % kAhead] = k_frag(sK, n);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
+        for (int r = 0; r < kRing; ++r) ring[r] = frag(No{}, -1, r);
+        __builtin_amdgcn_sched_barrier(0);
+        matrix_phase(No{}, Yes{}, -1);
+        take_mask_block(0, true, false);
+    }
+
+    // A wave computes on its first my_tiles tiles (all of them without a causal mask) and afterwards
+    // only keeps fetching its share of the remaining tiles and meeting the barriers.
+    for (int j = 0; j < my_tiles; ++j) {
+        // slot of tile j+dist: every wave is done with the tile it held (two barriers ago at the latest)
+        const bool issued = j + dist < n_tiles;
+        if (issued) issue_slice(j + dist, 0);
+        const int t0 = j * kBN;
+        constexpr bool active = true;
+
+        if (active) {
+            float x[32];
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                x[i] = st[0][i];
-                x[16 + i] = st[1][i];
+                x[i] = sc[0][i];
+                x[16 + i] = sc[1][i];
             }
-        }
-
-        if constexpr (kMaskViaLds) {
-            // this tile's mask values are in registers: the region can take the next block
-            if (active && j + 1 < my_tiles) {
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                issue_mask(j + 1);
-            }
-        }
-
-        if (active) {
             // scores in the log2 domain; without a mask the scale is folded into the exponent
             if constexpr (MASK != kNoMask) {
 #pragma unroll
@@ -207,10 +314,13 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
                     x[e] = key <= qrow ? x[e] : -INFINITY;
                 }
             }
-            float mx = x[0];
+            float mx = x[0], mx1 = x[16];  // two chains: a dependent maximum waits out the ALU latency
 #pragma unroll
-            for (int e = 1; e < 32; ++e) mx = fmaxf(mx, x[e]);
-            mx = fmaxf(mx, xor32(mx));
+            for (int e = 1; e < 16; ++e) {
+                mx = fmaxf(mx, x[e]);
+                mx1 = fmaxf(mx1, x[16 + e]);
+            }
+            mx = max_xor32(fmaxf(mx, mx1));
             if constexpr (MASK == kNoMask) mx *= c;
             // Lazy rescaling: m is the reference exponent of l and of the O accumulators, not
             // necessarily the running maximum. It is only moved (and O rescaled) when some row of
@@ -225,17 +335,46 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
                 for (int db = 0; db < DB; ++db)
 #pragma unroll
                     for (int i = 0; i < 16; ++i) oacc[db][i] *= alpha;
+                if constexpr (!DROPOUT) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) lacc[i] *= alpha;
+                }
             }
             const float m_use = m == -INFINITY ? 0.f : m;
+            // exponentials in four groups of eight keys (one B operand each); the remaining loads of the
+            // next tile and the first fragment reads of the matrix phase (tile j has been visible since
+            // the previous barrier) are issued between the groups, so that none of them queues
+            if (issued) issue_slice(j + dist, 1);
+            constexpr int kNow = kDefer ? 2 : 4;  // groups whose exponentials are taken here
 #pragma unroll
-            for (int e = 0; e < 32; ++e) {
-                if constexpr (MASK == kNoMask) x[e] = fast_exp2(fmaf(x[e], c, -m_use));
-                else x[e] = fast_exp2(x[e] - m_use);
+            for (int ks = 0; ks < kNow; ++ks) {
+#pragma unroll
+                for (int e = 8 * ks; e < 8 * ks + 8; ++e) {
+                    if constexpr (MASK == kNoMask) x[e] = fast_exp2(fmaf(x[e], c, -m_use));
+                    else x[e] = fast_exp2(x[e] - m_use);
+                }
+                if constexpr (!DROPOUT) pb[ks] = pack8<T>(&x[8 * ks]);
+                if (ks < 2 && issued) issue_slice(j + dist, 2 + ks);
+                if (ks < 2) {
+#pragma unroll
+                    for (int r = 3 * ks; r < 3 * ks + 3; ++r) ring[r] = frag(Yes{}, j, r);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
-            float psum = 0.f;
-            if constexpr (DROPOUT) {
+            if constexpr (kDefer) {
 #pragma unroll
-                for (int e = 0; e < 32; ++e) psum += x[e];
+                for (int e = 0; e < 16; ++e) xd[e] = x[16 + e];
+                m_def = m_use;
+            }
+            if constexpr (DROPOUT) {
+                // row sum before dropping, in fp32: four interleaved partial sums (a dependent add waits
+                // out the ALU latency)
+                float ps[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int e = 0; e < 32; ++e) ps[e & 3] += x[e];
+                l += (ps[0] + ps[1]) + (ps[2] + ps[3]);
+            }
+            if constexpr (DROPOUT) {
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb) {
                     // group g of key block kb: keys t0 + 32 kb + 8 g + 4 h .. +3; this lane generates g = lane % 4
@@ -251,41 +390,51 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
                         }
                 }
             }
-            // P as B operands; without dropout the row sum is taken from the rounded P that is
-            // actually multiplied with V, two values per instruction
-            u32x4 pb[4];
+            if constexpr (DROPOUT) {
+                // P as B operands
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                pb[ks] = pack8<T>(&x[8 * ks]);
-                if constexpr (!DROPOUT) {
-                    psum = Mma<T>::add_pair(pb[ks].x, psum);
-                    psum = Mma<T>::add_pair(pb[ks].y, psum);
-                    psum = Mma<T>::add_pair(pb[ks].z, psum);
-                    psum = Mma<T>::add_pair(pb[ks].w, psum);
-                }
-            }
-            l += psum;
-            // O^T += V^T P^T
-            {
-                u32x4 vring[kPvAhead];
-#pragma unroll
-                for (int s = 0; s < kPvAhead; ++s)
-                    vring[s] = v_frag(sV, s);
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int s = 0; s < kPvSteps; ++s) {
-                    oacc[s % DB] = Mma<T>::run(vring[s % kPvAhead], pb[s / DB], oacc[s % DB]);
-                    if (s + kPvAhead < kPvSteps) {
-                        const int n = s + kPvAhead;
-                        vring[s % kPvAhead] = v_frag(sV, n);
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-                }
+                for (int ks = 0; ks < 4; ++ks) pb[ks] = pack8<T>(&x[8 * ks]);
             }
         }
-    }
+        static_assert(kRing == 6, "the softmax phase requests fragments 0..5");
 
-    l += xor32(l);
+        const bool with_s = j + 1 < my_tiles;
+        // tile j+dist-1 has landed (the next mask block and the newest tile may still be in flight);
+        // after the barrier it is visible to every wave, and the partner group changes phase. The
+        // fragment reads stay in flight across the barrier: nothing overwrites their slot before the
+        // barrier after next.
+        wait_loads(kMaskViaLds && with_s, issued);
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+
+        if (active) {
+            // (a wave's last tile also runs the S^T steps, on whatever the next slot holds: the result
+            // is never used, and one instruction stream serves every tile)
+            if (with_s) load_mask(j + 1);
+            // the few instructions of this phase go first, so that the matrix pipe never waits for an
+            // issue slot behind the partner's vector work
+            __builtin_amdgcn_s_setprio(2);
+            matrix_phase(Yes{}, Yes{}, j);
+            __builtin_amdgcn_s_setprio(0);
+            if (with_s) take_mask_block(j + 1, false, issued);
+        }
+        if constexpr (kPingPong) {
+            __builtin_amdgcn_sched_barrier(0);
+            lds_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    for (int j = my_tiles; j < n_tiles; ++j) {
+        const bool issued = j + dist < n_tiles;
+        if (issued) issue_tile(j + dist);
+        wait_loads(false, issued);
+        lds_barrier();
+        if constexpr (kPingPong) lds_barrier();
+    }
+    if (kPingPong && group == 0) lds_barrier();  // group 1 is still in its last matrix phase
+
+    l = DROPOUT ? sum_xor32(l) : lacc[0];
     const float inv = 1.f / l;
     // every wave is out of the loop: the ring can serve as the waves' private transposition patches
     lds_barrier();
