@@ -627,28 +627,45 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
         if (lt == 0 && n_local > 1) TRI_WAIT_VMCNT(kLoadsPerTile);
         else TRI_WAIT_VMCNT(0);
         lds_barrier();
+    };
+    // (after the barrier every wave is done with tile lt-2, whose slot tile lt+1 takes)
+    auto issue_next = [&](int lt) {
         if (lt >= 1 && lt + 1 < n_local) issue_tile(t_begin + lt + 1);
     };
-    // score step: P and dS of query block `member` of local tile lt against this pair's keys
-    auto score = [&](int lt) {
+    // A step is split once more, so that the matrix pipe and the vector ALU of the SIMD are both busy:
+    //   first part:  the scoring member runs its 16 MFMAs (S and dP); the accumulating member exchanges
+    //                P and dS through the LDS slots and requests its first fragments;
+    //   second part: the scoring member does the softmax arithmetic; the accumulating member runs its
+    //                16 MFMAs.
+    // (Both members issuing MFMAs at once, and the arithmetic afterwards with an idle matrix pipe, cost
+    // more than twice the time.) part_barrier() separates the parts; it does not wait for LDS reads in
+    // flight, which the second part consumes.
+    auto part_barrier = [&]() {
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // The state a step carries from its first part to its second. Every variable is assigned in every
+    // first part (zeros on the idle paths), so that none of them stays live around the loop.
+    f32x16 sc_s, sc_dp;                      // scores
+    f32x4 sc_lse[4];                         // lse of this lane's 16 rows
+    // (deeper fragment rings and delta fetched ahead like lse were measured: no gain, 14 more registers)
+    constexpr bool kRoomy = false;
+    f32x4 sc_dlt[kRoomy ? 4 : 1];            // delta of the same rows
+    u32x4 own_p[2], own_s[2], pp[2], ps[2];  // B operands of the accumulation
+    constexpr int kAccSteps = 8 * DH, kAccRing = kRoomy ? 6 : 4;
+    u32x4 tf[kAccRing];                      // first transposed fragments of the accumulation
+    // score step, first part: S and dP of query block `member` of local tile lt against this pair's keys
+    auto score_mfma = [&](int lt, bool issue) {
         const int j = t_begin + lt;
         const int rb = j * kBN + 32 * member;
+        const char* sQ = smem + ((lt < n_local ? lt : 0) % kStages) * kStageBytes;
+        const char* sG = sQ + Tile::kBytes;
+        const float* sLse = reinterpret_cast<const float*>(sG + Tile::kBytes);
         if (lt < n_local && (!CAUSAL || rb + 31 >= wkey0)) {
-            const char* sQ = smem + (lt % kStages) * kStageBytes;
-            const char* sG = sQ + Tile::kBytes;
-            const float* sLse = reinterpret_cast<const float*>(sG + Tile::kBytes);
-            const float* sDelta = sLse + kBN;
-            const bool diag = CAUSAL && rb < wkey0 + 31;
-            float mk[MASK != kNoMask ? 16 : 1];
-            if constexpr (MASK != kNoMask) {
-                const int64_t mbase = b * p.ms[0] + hd * p.ms[1] + key;
-#pragma unroll
-                for (int i = 0; i < 16; ++i)
-                    mk[i] = mask_at<T, MASK>(p.mask, mbase + static_cast<int64_t>(rb + c_row(i, h)) * p.ms[2]);
-            }
             const int qoff = 32 * member * Tile::kRowBytes;
             // row fragments of Q, then of dO, through a ring of kRing reads in flight
-            constexpr int kRing = 4;
+            constexpr int kRing = kRoomy ? 6 : 4;
             auto row_frag = [&](int n) {
                 return lds_read16(n < KK ? sQ : sG, (row_off0 ^ ((n % KK) << 5)) + qoff);
             };
@@ -656,6 +673,11 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
 #pragma unroll
             for (int n = 0; n < kRing; ++n) fr[n] = row_frag(n);
             __builtin_amdgcn_sched_barrier(0);
+            // the loads of the next tile go out while the first fragments are on their way (a load
+            // instruction holds the wave until the memory pipeline takes it)
+            if (issue) issue_next(lt);
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_setprio(2);
             f32x16 s = zero16(), dp = zero16();
 #pragma unroll
             for (int n = 0; n < 2 * KK; ++n) {
@@ -664,16 +686,55 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
                 if (n + kRing < 2 * KK) fr[n % kRing] = row_frag(n + kRing);
                 __builtin_amdgcn_sched_barrier(0);
             }
+            __builtin_amdgcn_s_setprio(0);
+            sc_s = s;
+            sc_dp = dp;
+        } else {
+            if (issue) issue_next(lt);
+            sc_s = zero16();
+            sc_dp = zero16();
+        }
+        // requested now, used in the second part (harmless where the step is idle)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) sc_lse[g] = *reinterpret_cast<const f32x4*>(sLse + 32 * member + 8 * g + 4 * h);
+        if constexpr (kRoomy) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) sc_dlt[g] = *reinterpret_cast<const f32x4*>(sLse + kBN + 32 * member + 8 * g + 4 * h);
+        }
+    };
+    // score step, second part: P and dS from the scores, packed as B operands
+    auto score_valu = [&](int lt) {
+        const int j = t_begin + lt;
+        const int rb = j * kBN + 32 * member;
+        if (lt < n_local && (!CAUSAL || rb + 31 >= wkey0)) {
+            const char* sQ = smem + (lt % kStages) * kStageBytes;
+            const char* sG = sQ + Tile::kBytes;
+            const float* sDelta = reinterpret_cast<const float*>(sG + Tile::kBytes) + kBN;
+            const bool diag = CAUSAL && rb < wkey0 + 31;
+            const f32x16 s = sc_s, dp = sc_dp;
+            float mk[MASK != kNoMask ? 16 : 1];
+            if constexpr (MASK != kNoMask) {
+                const int64_t mbase = b * p.ms[0] + hd * p.ms[1] + key;
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    mk[i] = mask_at<T, MASK>(p.mask, mbase + static_cast<int64_t>(rb + c_row(i, h)) * p.ms[2]);
+            }
             Philox4 mine;  // the block of rows rb + 8 (lane % 4) + 4 h .. +3: this lane's share of the quad's four
             if constexpr (DROPOUT) mine = dropout_block(p, bh, (rb + 8 * (lane & 3) + 4 * h) >> 2, key >> 2);
 #pragma unroll
             for (int gg = 0; gg < 2; ++gg) {  // eight rows at a time, packed as soon as they are done
                 float pr[8], ds[8];
+                f32x4 dlt4[2];
+#pragma unroll
+                for (int g2 = 0; g2 < 2; ++g2) {
+                    if constexpr (kRoomy) dlt4[g2] = sc_dlt[2 * gg + g2];
+                    else dlt4[g2] = *reinterpret_cast<const f32x4*>(sDelta + 32 * member + 8 * (2 * gg + g2) + 4 * h);
+                }
 #pragma unroll
                 for (int g2 = 0; g2 < 2; ++g2) {
                     const int g = 2 * gg + g2;
-                    f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + 32 * member + 8 * g + 4 * h);
-                    const f32x4 d4 = *reinterpret_cast<const f32x4*>(sDelta + 32 * member + 8 * g + 4 * h);
+                    f32x4 l4 = sc_lse[g];
+                    const f32x4 d4 = dlt4[g2];
                     if constexpr (MASK != kNoMask) {
 #pragma unroll
                         for (int bb = 0; bb < 4; ++bb) l4[bb] = l4[bb] == -INFINITY ? INFINITY : l4[bb];
@@ -711,10 +772,21 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
             for (int g = 0; g < 2; ++g) cur_p[g] = cur_s[g] = u32x4{0, 0, 0, 0};
         }
     };
-    // accumulation step: publish the latest scores, then add local tile lt to this member's half of
-    // the head dimension for both query blocks
-    auto accumulate = [&](int lt) {
-        u32x4 own_p[2], own_s[2];
+    // accumulation step, first part: publish the latest scores, fetch the partner's and the first
+    // transposed fragments. Second part: add local tile lt to this member's half of the head dimension
+    // for both query blocks: 8 DH MFMAs in the order (query block, K-step, dV^T or dK^T, column block),
+    // their A operands through one ring of fragments.
+    auto acc_frag = [&](int lt, int n) {
+        const char* sQ = smem + (lt % kStages) * kStageBytes;
+        const char* sG = sQ + Tile::kBytes;
+        const int d = n % DH, which = (n / DH) % 2, g = (n / (2 * DH)) % 2, qb = n / (4 * DH);
+        const int db = DH * member + d;
+        return Tile::tr_frag(which ? sQ : sG, tr_off0 ^ (db << 6), tr_off1 ^ (db << 6), 2 * qb + g);
+    };
+    auto acc_on = [&](int lt) {
+        return lt >= 0 && lt < n_local && (!CAUSAL || (t_begin + lt) * kBN + kBN - 1 >= wkey0);
+    };
+    auto acc_prep = [&](int lt) {
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
             if (member == 0) {  // LDS operations of one wave complete in order: read, then overwrite
@@ -731,40 +803,28 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
             *reinterpret_cast<u32x4*>(my_xch + g * 1024) = cur_p[g];
             *reinterpret_cast<u32x4*>(my_xch + (2 + g) * 1024) = cur_s[g];
         }
-        const int j = t_begin + lt;
-        const int r0 = j * kBN;
-        if (lt >= 0 && lt < n_local && (!CAUSAL || r0 + kBN - 1 >= wkey0)) {
-            const char* sQ = smem + (lt % kStages) * kStageBytes;
-            const char* sG = sQ + Tile::kBytes;
-            u32x4 pp[2], ps[2];  // the partner's P and dS
+        // (unconditional reads: harmless where the step is idle)
 #pragma unroll
-            for (int g = 0; g < 2; ++g) {
-                pp[g] = *reinterpret_cast<const u32x4*>(peer_xch + g * 1024);
-                ps[g] = *reinterpret_cast<const u32x4*>(peer_xch + (2 + g) * 1024);
+        for (int g = 0; g < 2; ++g) {  // the partner's P and dS
+            pp[g] = *reinterpret_cast<const u32x4*>(peer_xch + g * 1024);
+            ps[g] = *reinterpret_cast<const u32x4*>(peer_xch + (2 + g) * 1024);
+        }
+        const int lt_safe = lt >= 0 && lt < n_local ? lt : 0;
+#pragma unroll
+        for (int n = 0; n < kAccRing; ++n) tf[n] = acc_frag(lt_safe, n);
+    };
+    auto acc_mfma = [&](int lt) {
+        if (acc_on(lt)) {
+            __builtin_amdgcn_s_setprio(2);
+#pragma unroll
+            for (int n = 0; n < kAccSteps; ++n) {
+                const int d = n % DH, which = (n / DH) % 2, g = (n / (2 * DH)) % 2, qb = n / (4 * DH);
+                if (which == 0) dv[d] = Mma<T>::run(tf[n % kAccRing], qb == member ? own_p[g] : pp[g], dv[d]);
+                else dk[d] = Mma<T>::run(tf[n % kAccRing], qb == member ? own_s[g] : ps[g], dk[d]);
+                if (n + kAccRing < kAccSteps) tf[n % kAccRing] = acc_frag(lt, n + kAccRing);
+                __builtin_amdgcn_sched_barrier(0);
             }
-#pragma unroll
-            for (int qb = 0; qb < 2; ++qb) {
-#pragma unroll
-                for (int g = 0; g < 2; ++g) {
-                    const u32x4 bp = qb == member ? own_p[g] : pp[g];
-                    const u32x4 bs = qb == member ? own_s[g] : ps[g];
-                    u32x4 tf[DH];
-#pragma unroll
-                    for (int d = 0; d < DH; ++d) {
-                        const int db = DH * member + d;
-                        tf[d] = Tile::tr_frag(sG, tr_off0 ^ (db << 6), tr_off1 ^ (db << 6), 2 * qb + g);
-                    }
-#pragma unroll
-                    for (int d = 0; d < DH; ++d) {
-                        const int db = DH * member + d;
-                        dv[d] = Mma<T>::run(tf[d], bp, dv[d]);
-                        tf[d] = Tile::tr_frag(sQ, tr_off0 ^ (db << 6), tr_off1 ^ (db << 6), 2 * qb + g);
-                    }
-#pragma unroll
-                    for (int d = 0; d < DH; ++d) dk[d] = Mma<T>::run(tf[d], bs, dk[d]);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            }
+            __builtin_amdgcn_s_setprio(0);
         }
     };
 
@@ -772,17 +832,26 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
 #pragma unroll 1
         for (int lt = 0; lt <= n_local; ++lt) {
             open_even_step(lt);
-            score(lt);
+            score_mfma(lt, true);
+            part_barrier();
+            score_valu(lt);
             lds_barrier();
-            accumulate(lt - 1);
+            acc_prep(lt - 1);
+            part_barrier();
+            acc_mfma(lt - 1);
         }
     } else {
 #pragma unroll 1
         for (int lt = 0; lt <= n_local; ++lt) {
             open_even_step(lt);
-            accumulate(lt - 1);
+            issue_next(lt);
+            acc_prep(lt - 1);
+            part_barrier();
+            acc_mfma(lt - 1);
             lds_barrier();
-            score(lt);
+            score_mfma(lt, false);
+            part_barrier();
+            score_valu(lt);
         }
     }
 
