@@ -224,7 +224,8 @@ def test_dropout_mask_bits_match_oracle(device):
         assert (keep.cpu().numpy().reshape(rows, cols).astype(bool) == want).all()
 
 
-@pytest.mark.parametrize("dtype,S,D", [(torch.float32, 64, 32), (torch.bfloat16, 256, 128), (torch.float16, 128, 64)])
+@pytest.mark.parametrize("dtype,S,D", [(torch.float32, 64, 32), (torch.bfloat16, 256, 128), (torch.float16, 128, 64),
+                                       (torch.bfloat16, 512, 64), (torch.float16, 512, 128)])
 @pytest.mark.parametrize("p", [0.1, 0.5])
 def test_dropout_forward_backward(dtype, S, D, p, device):
     q, k, v, d_o = _gen((2, 2, S, D), 61, dtype)

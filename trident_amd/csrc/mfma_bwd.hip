@@ -10,6 +10,8 @@
 // In both, the lane index is the row that owns the accumulators (query row resp. key), the
 // stationary operands (Q,dO resp. K,V) stay in registers as MFMA B operands, and P / dS go
 // from the accumulators of one MFMA to the B operand of the next without leaving registers.
+#include <type_traits>
+
 #include "launch.hpp"
 #include "mfma_common.hpp"
 
@@ -225,6 +227,226 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
             for (int i = 0; i < 2 * DB; ++i) acc[i % DB] = Mma<T>::run(tf[i], bop[i / DB], acc[i % DB]);
         }
     }
+
+    // every wave is out of the loop: the ring can serve as the waves' private transposition patches
+    lds_barrier();
+    {
+        using Store = RowBlockStore<T, DB>;
+        static_assert(NW * Store::kPatchBytes <= kStages * kStageBytes, "patches must fit into the ring");
+        char* out0 = static_cast<char*>(p.dq) + (b * p.dqs[0] + hd * p.dqs[1] + static_cast<int64_t>(wrow0) * p.dqs[2]) * 2;
+        const float sc = p.scale;
+        Store::run(acc, [sc](float x) { return x * sc; }, smem + wave * Store::kPatchBytes, out0, p.dqs[2] * 2, lane);
+    }
+}
+
+// ------------------------------------------------------------------ dQ, phased (8 waves, no mask)
+// Same data flow and tile ring as above, restructured so that the two waves of a SIMD (w and w+4)
+// never do the same kind of work at once. Per 64-key tile a wave runs a vector phase (P and dS of the
+// tile from its S^T and dP^T, packed as B operands) and a matrix phase (dQ^T += K^T dS^T of this
+// tile, then S^T and dP^T of the next one: 6 D / 16 MFMAs through one ring of LDS fragments), with a
+// workgroup barrier after each; waves 4-7 run one phase behind waves 0-3. Tile loads are issued at
+// the top of the vector phase (two tiles ahead in waves 0-3, three in waves 4-7, which start their
+// phase later) and awaited before its barrier.
+template <typename T, int D, bool CAUSAL, bool DROPOUT>
+__global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p) {
+    using Tile = SwzTile<D>;
+    constexpr int NW = 8;
+    constexpr int kRows = 32 * NW;
+    constexpr int kStages = 4;
+    constexpr int kStageBytes = 2 * Tile::kBytes;  // K tile, V tile
+    constexpr int KK = D / 16;
+    constexpr int DB = D / 32;
+    constexpr int kBlocksPerWave = 2 * Tile::kBlocks / NW;
+    constexpr int kPerOperand = Tile::kBlocks / NW;
+    constexpr int kRowStep = NW * Tile::kRowsPerBlock;
+    static_assert(kRowStep % 16 == 0 && 2 * kPerOperand == kBlocksPerWave, "block assignment");
+    constexpr int kDqSteps = 4 * DB;           // MFMAs of dQ^T per tile
+    constexpr int kSteps = kDqSteps + 4 * KK;  // + S^T and dP^T of the next tile
+    constexpr int kRing = 6;
+    static_assert(kRing <= kDqSteps, "the vector phase requests dQ fragments only");
+    __shared__ __attribute__((aligned(1024))) char smem[kStages * kStageBytes];
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+    int bh, qt;
+    map_block(blockIdx.x, p.B * p.H, p.S / kRows, CAUSAL ? kHeavyLast : kUniformTiles, &bh, &qt);
+    const int b = bh / p.H, hd = bh % p.H;
+    const int q0 = qt * kRows;
+    const int wrow0 = q0 + 32 * wave;
+    const int qrow = wrow0 + l32;
+
+    const char* qrowp = static_cast<const char*>(p.q) + (b * p.qs[0] + hd * p.qs[1] + static_cast<int64_t>(qrow) * p.qs[2]) * 2;
+    const char* gorowp = static_cast<const char*>(p.d_o) + (b * p.dos[0] + hd * p.dos[1] + static_cast<int64_t>(qrow) * p.dos[2]) * 2;
+    const char* kbase = static_cast<const char*>(p.k) + (b * p.ks[0] + hd * p.ks[1]) * 2;
+    const char* vbase = static_cast<const char*>(p.v) + (b * p.vs[0] + hd * p.vs[1]) * 2;
+    const int64_t krow_bytes = p.ks[2] * 2, vrow_bytes = p.vs[2] * 2;
+
+    u32x4 qf[KK], gf[KK];
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+        qf[kk] = *reinterpret_cast<const u32x4*>(qrowp + (2 * kk + h) * 16);
+        gf[kk] = *reinterpret_cast<const u32x4*>(gorowp + (2 * kk + h) * 16);
+    }
+    float lse = p.lse[static_cast<int64_t>(bh) * p.S + qrow];
+    if (lse == -INFINITY) lse = INFINITY;  // fully masked row: every probability is 0
+    const float dlt = p.delta[static_cast<int64_t>(bh) * p.S + qrow];
+    const float c = p.scale_log2;
+
+    f32x16 acc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) acc[db] = zero16();
+
+    const int n_tiles = CAUSAL ? (q0 + kRows) / kBN : p.S / kBN;     // tiles the workgroup streams
+    const int my_tiles = CAUSAL ? (wrow0 + 31) / kBN + 1 : n_tiles;  // tiles with keys visible to this wave
+
+    // A wave fetches blocks wave, wave + NW, ... of the K tile and of the V tile: their rows are a
+    // multiple of 16 apart, so one per-lane source offset serves all of them.
+    const uint32_t koff = static_cast<uint32_t>(Tile::src_off(wave, lane, krow_bytes));
+    const uint32_t voff = static_cast<uint32_t>(Tile::src_off(wave, lane, vrow_bytes));
+    auto issue_tile = [&](int t) {
+        char* stage = smem + (t % kStages) * kStageBytes + wave * 1024;
+#pragma unroll
+        for (int i = 0; i < kPerOperand; ++i)
+            lds_direct_load16(kbase + (static_cast<int64_t>(t) * kBN + i * kRowStep) * krow_bytes, koff, stage + i * NW * 1024);
+#pragma unroll
+        for (int i = 0; i < kPerOperand; ++i)
+            lds_direct_load16(vbase + (static_cast<int64_t>(t) * kBN + i * kRowStep) * vrow_bytes, voff,
+                              stage + Tile::kBytes + i * NW * 1024);
+    };
+    const int group = wave >> 2;
+    const int dist = 2 + group;
+    const int n_first = min(dist, n_tiles);
+    issue_tile(0);
+    if (n_first > 1) issue_tile(1);
+    if (n_first > 2) issue_tile(2);
+    // (the row fragments were requested before the tiles, so both latencies overlap)
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+        settle(qf[kk]);
+        settle(gf[kk]);
+    }
+    settle(lse);
+    settle(dlt);
+
+    const int row_off0 = Tile::off(l32, h);
+    const int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
+
+    // fragment n of the matrix phase of tile t: n < kDqSteps: K^T of tile t (column block n % DB, K-step
+    // n / DB); then the K rows (key block 0, 1) and the V rows (key block 0, 1) of tile t + 1
+    auto frag = [&](int t, int n) {
+        if (n < kDqSteps) {
+            const char* sK = smem + ((t + kStages) % kStages) * kStageBytes;
+            return Tile::tr_frag(sK, tr_off0 ^ ((n % DB) << 6), tr_off1 ^ ((n % DB) << 6), n / DB);
+        }
+        const int m = n - kDqSteps;
+        const char* sT = smem + ((t + 1) % kStages) * kStageBytes + (m < 2 * KK ? 0 : Tile::kBytes);
+        return lds_read16(sT, (row_off0 ^ ((m % KK) << 5)) + 32 * ((m / KK) & 1) * Tile::kRowBytes);
+    };
+    f32x16 st[2], dpt[2];  // S^T and dP^T of the current tile (two key blocks)
+    u32x4 bop[4];          // dS^T of the current tile as B operands
+    u32x4 ring[kRing];
+    auto matrix_phase = [&](auto with_dq, int t) {
+        constexpr int first = decltype(with_dq)::value ? 0 : kDqSteps;
+        f32x16 s_new[2] = {zero16(), zero16()}, dp_new[2] = {zero16(), zero16()};
+#pragma unroll
+        for (int n = first; n < kSteps; ++n) {
+            const int slot = (n - first) % kRing;
+            const int m = n - kDqSteps;
+            if (n < kDqSteps) acc[n % DB] = Mma<T>::run(ring[slot], bop[n / DB], acc[n % DB]);
+            else if (m < 2 * KK) s_new[m / KK] = Mma<T>::run(ring[slot], qf[m % KK], s_new[m / KK]);
+            else dp_new[(m / KK) & 1] = Mma<T>::run(ring[slot], gf[m % KK], dp_new[(m / KK) & 1]);
+            if (n + kRing < kSteps) ring[slot] = frag(t, n + kRing);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        st[0] = s_new[0]; st[1] = s_new[1];
+        dpt[0] = dp_new[0]; dpt[1] = dp_new[1];
+    };
+    using Yes = std::integral_constant<bool, true>;
+    using No = std::integral_constant<bool, false>;
+    auto wait_tile = [&](bool newest_in_flight) {
+        if (newest_in_flight) TRI_WAIT_VMCNT(kBlocksPerWave);
+        else TRI_WAIT_VMCNT(0);
+    };
+
+    // tile 0 has landed and is visible to all waves
+    if (n_first == 3) TRI_WAIT_VMCNT(2 * kBlocksPerWave);
+    else if (n_first == 2) TRI_WAIT_VMCNT(kBlocksPerWave);
+    else TRI_WAIT_VMCNT(0);
+    lds_barrier();
+    if (group == 1) {
+        // group 1 starts one phase late; group 0 reads tile 1 in its first matrix phase
+        if (n_first == 3) TRI_WAIT_VMCNT(kBlocksPerWave);
+        else TRI_WAIT_VMCNT(0);
+        lds_barrier();
+    }
+    {
+#pragma unroll
+        for (int r = 0; r < kRing; ++r) ring[r] = frag(-1, kDqSteps + r);
+        __builtin_amdgcn_sched_barrier(0);
+        matrix_phase(No{}, -1);
+    }
+
+    for (int t = 0; t < my_tiles; ++t) {
+        const bool issued = t + dist < n_tiles;
+        if (issued) issue_tile(t + dist);
+        // ---- vector phase: P and dS of the tile
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            const int key0 = t * kBN + 32 * kb;
+            const bool diag = CAUSAL && key0 + 31 > wrow0;
+            float ds[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                float pr = fast_exp2(fmaf(st[kb][i], c, -lse));
+                if (diag) pr = key0 + c_row(i, h) <= qrow ? pr : 0.f;
+                ds[i] = pr;
+            }
+            f32x16 dpv = dpt[kb];
+            if constexpr (DROPOUT) {
+                const Philox4 mine = dropout_block(p, bh, qrow >> 2, (key0 + 8 * (lane & 3) + 4 * h) >> 2);
+                uint32_t w[4];
+                quad_row_words(mine, lane, w);
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+#pragma unroll
+                    for (int bb = 0; bb < 4; ++bb) {
+                        const bool keep = static_cast<int>((w[g] >> (8 * bb)) & 0xffu) >= p.thr8;
+                        dpv[4 * g + bb] = keep ? dpv[4 * g + bb] * p.zscale : 0.f;
+                    }
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) ds[i] *= dpv[i] - dlt;
+            bop[2 * kb + 0] = pack8<T>(&ds[0]);
+            bop[2 * kb + 1] = pack8<T>(&ds[8]);
+        }
+        // the first fragments of the matrix phase (K^T of this tile, visible since the previous barrier)
+#pragma unroll
+        for (int r = 0; r < kRing; ++r) ring[r] = frag(t, r);
+        // tile t + dist - 1 has landed (the newest one may still be in flight); after the barrier it is
+        // visible to every wave, and the partner group changes phase
+        wait_tile(issued);
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- matrix phase (a wave's last tile also runs the S^T / dP^T steps, on whatever the next slot
+        // holds: the result is never used)
+        __builtin_amdgcn_s_setprio(2);
+        matrix_phase(Yes{}, t);
+        __builtin_amdgcn_s_setprio(0);
+        __builtin_amdgcn_sched_barrier(0);
+        lds_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // afterwards a wave only keeps fetching its share of the remaining tiles and meeting the barriers
+    for (int t = my_tiles; t < n_tiles; ++t) {
+        const bool issued = t + dist < n_tiles;
+        if (issued) issue_tile(t + dist);
+        wait_tile(issued);
+        lds_barrier();
+        lds_barrier();
+    }
+    if (group == 0) lds_barrier();  // group 1 is still in its last matrix phase
 
     // every wave is out of the loop: the ring can serve as the waves' private transposition patches
     lds_barrier();
@@ -883,6 +1105,20 @@ int launch_dq_waves(const KParams& p, hipStream_t stream) {
 template <typename T, int D, bool CAUSAL, int MASK>
 int launch_dq_dropout(const KParams& p, hipStream_t stream) {
     // 8 waves (256 query rows) when the sequence allows it, else 4 waves (128 rows)
+    if constexpr (MASK == kNoMask) {
+        // the phased kernel (with dropout at D = 128 it would not fit its registers)
+        if (p.S % 256 == 0 && (D == 64 || p.thr8 <= 0)) {
+            const dim3 grid(p.B * p.H * (p.S / 256)), block(512);
+            if constexpr (D == 64) {
+                if (p.thr8 > 0) {
+                    hipLaunchKernelGGL((mfma_dq_phased_kernel<T, D, CAUSAL, true>), grid, block, 0, stream, p);
+                    return static_cast<int>(hipGetLastError());
+                }
+            }
+            hipLaunchKernelGGL((mfma_dq_phased_kernel<T, D, CAUSAL, false>), grid, block, 0, stream, p);
+            return static_cast<int>(hipGetLastError());
+        }
+    }
     if (p.S % 256 == 0) return launch_dq_waves<T, D, 8, CAUSAL, MASK>(p, stream);
     return launch_dq_waves<T, D, 4, CAUSAL, MASK>(p, stream);
 }
