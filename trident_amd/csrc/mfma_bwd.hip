@@ -871,11 +871,11 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
     // first part (zeros on the idle paths), so that none of them stays live around the loop.
     f32x16 sc_s, sc_dp;                      // scores
     f32x4 sc_lse[4];                         // lse of this lane's 16 rows
-    // (deeper fragment rings and delta fetched ahead like lse were measured: no gain, 14 more registers)
+    // (fetching delta ahead like lse, and deeper fragment rings, were measured: no gain)
     constexpr bool kRoomy = false;
     f32x4 sc_dlt[kRoomy ? 4 : 1];            // delta of the same rows
     u32x4 own_p[2], own_s[2], pp[2], ps[2];  // B operands of the accumulation
-    constexpr int kAccSteps = 8 * DH, kAccRing = kRoomy ? 6 : 4;
+    constexpr int kAccSteps = 8 * DH, kAccRing = 4;
     u32x4 tf[kAccRing];                      // first transposed fragments of the accumulation
     // score step, first part: S and dP of query block `member` of local tile lt against this pair's keys
     auto score_mfma = [&](int lt, bool issue) {
@@ -887,7 +887,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
         if (lt < n_local && (!CAUSAL || rb + 31 >= wkey0)) {
             const int qoff = 32 * member * Tile::kRowBytes;
             // row fragments of Q, then of dO, through a ring of kRing reads in flight
-            constexpr int kRing = kRoomy ? 6 : 4;
+            constexpr int kRing = 4;
             auto row_frag = [&](int n) {
                 return lds_read16(n < KK ? sQ : sG, (row_off0 ^ ((n % KK) << 5)) + qoff);
             };
