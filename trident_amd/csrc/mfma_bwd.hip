@@ -850,7 +850,9 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
         else TRI_WAIT_VMCNT(0);
         lds_barrier();
     };
-    // (after the barrier every wave is done with tile lt-2, whose slot tile lt+1 takes)
+    // (after the barrier every wave is done with tile lt-2, whose slot tile lt+1 takes; a member issues
+    // its share of the loads at the start of its accumulation step, the part of a tile in which it
+    // would otherwise only wait: a load instruction holds the wave until the memory pipeline takes it)
     auto issue_next = [&](int lt) {
         if (lt >= 1 && lt + 1 < n_local) issue_tile(t_begin + lt + 1);
     };
@@ -878,7 +880,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
     constexpr int kAccSteps = 8 * DH, kAccRing = 4;
     u32x4 tf[kAccRing];                      // first transposed fragments of the accumulation
     // score step, first part: S and dP of query block `member` of local tile lt against this pair's keys
-    auto score_mfma = [&](int lt, bool issue) {
+    auto score_mfma = [&](int lt) {
         const int j = t_begin + lt;
         const int rb = j * kBN + 32 * member;
         const char* sQ = smem + ((lt < n_local ? lt : 0) % kStages) * kStageBytes;
@@ -895,10 +897,6 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
 #pragma unroll
             for (int n = 0; n < kRing; ++n) fr[n] = row_frag(n);
             __builtin_amdgcn_sched_barrier(0);
-            // the loads of the next tile go out while the first fragments are on their way (a load
-            // instruction holds the wave until the memory pipeline takes it)
-            if (issue) issue_next(lt);
-            __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_setprio(2);
             f32x16 s = zero16(), dp = zero16();
 #pragma unroll
@@ -912,7 +910,6 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
             sc_s = s;
             sc_dp = dp;
         } else {
-            if (issue) issue_next(lt);
             sc_s = zero16();
             sc_dp = zero16();
         }
@@ -1054,10 +1051,11 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
 #pragma unroll 1
         for (int lt = 0; lt <= n_local; ++lt) {
             open_even_step(lt);
-            score_mfma(lt, true);
+            score_mfma(lt);
             part_barrier();
             score_valu(lt);
             lds_barrier();
+            issue_next(lt);  // in the part where this member only waits for the partner's MFMAs
             acc_prep(lt - 1);
             part_barrier();
             acc_mfma(lt - 1);
@@ -1071,7 +1069,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
             part_barrier();
             acc_mfma(lt - 1);
             lds_barrier();
-            score_mfma(lt, false);
+            score_mfma(lt);
             part_barrier();
             score_valu(lt);
         }
