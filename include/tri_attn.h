@@ -124,8 +124,10 @@ int tri_attn_bwd_dkdv(const TriAttnArgs* args);
  * Reads q,k,v,d_o,lse,delta[,mask]; writes dq[, dmask]. */
 int tri_attn_bwd_dq(const TriAttnArgs* args);
 
-/* The whole backward in launch order: bwd_delta, bwd_dkdv, bwd_dq
- * (trident/operation/attention.py:137-202). */
+/* The whole backward (trident/operation/attention.py:137-202): the results of bwd_delta, bwd_dkdv and
+ * bwd_dq called in that order, written to delta, dk, dv, dq[, dmask]. The library may launch fewer
+ * kernels and in another order: without a mask, for sequence lengths that are multiples of 256 (and
+ * without dropout at D = 128) the dQ kernel computes delta on its way and runs before dK/dV. */
 int tri_attn_bwd(const TriAttnArgs* args);
 
 /* Debug / parity helper with no counterpart in the reference (its dropout stream is unpinned):

@@ -298,6 +298,48 @@ def test_lengths_that_are_not_powers_of_two(dtype, S, D, variant, device):
     _abi_case(device, dtype, S, D, variant, 300 + S + D)
 
 
+# ------------------------------------------------------------------ the combined backward entry point
+@pytest.mark.parametrize("S,D,causal,p", [(512, 128, True, 0.0), (256, 64, False, 0.0), (512, 64, True, 0.25),
+                                          (256, 128, True, 0.25), (384, 128, True, 0.0)])
+def test_combined_backward_matches_the_three_calls(S, D, causal, p, device):
+    """tri_attn_bwd may fold the delta pre-pass into the dQ kernel and reorder the launches; its
+    results must be those of delta, dK/dV and dQ called one after the other."""
+    import ctypes
+    from trident_amd import _lib, operation
+    lib = _lib.lib()
+    q, k, v, d_o = [x.to(device) for x in _gen((2, 2, S, D), 400 + S + D, torch.bfloat16)]
+    o = torch.empty_like(q)
+    lse = torch.empty(2, 2, S, device=device, dtype=torch.float32)
+    outs = []
+    for combined in (False, True):
+        delta = torch.full_like(lse, float("nan"))
+        dq, dk, dv = [torch.full_like(q, float("nan")) for _ in range(3)]
+        args = operation._base_args(q, None, p, causal, 1.0 / math.sqrt(D), 99 if p > 0 else 0, 0)
+        for name, t, field in [("q", q, "q_stride"), ("k", k, "k_stride"), ("v", v, "v_stride"), ("o", o, "o_stride"),
+                               ("d_o", d_o, "do_stride"), ("dq", dq, "dq_stride"), ("dk", dk, "dk_stride"),
+                               ("dv", dv, "dv_stride")]:
+            operation._fill(args, name, t, field)
+        operation._fill(args, "lse", lse)
+        operation._fill(args, "delta", delta)
+        ref = ctypes.byref(args)
+        _lib.check(lib.tri_attn_fwd(ref))
+        if combined:
+            _lib.check(lib.tri_attn_bwd(ref))
+        else:
+            _lib.check(lib.tri_attn_bwd_delta(ref))
+            _lib.check(lib.tri_attn_bwd_dkdv(ref))
+            _lib.check(lib.tri_attn_bwd_dq(ref))
+        torch.cuda.synchronize()
+        outs.append((delta.clone(), dq.clone(), dk.clone(), dv.clone()))
+    (d0, q0, k0, v0), (d1, q1, k1, v1) = outs
+    assert not torch.isnan(d1).any()
+    # delta: the same fp32 products summed in another order
+    assert (d0 - d1).abs().max().item() <= 1e-4 * max(1.0, d0.abs().max().item())
+    for a, b_ in ((q0, q1), (k0, k1), (v0, v1)):
+        assert not torch.isnan(b_.float()).any()
+        assert (a.float() - b_.float()).abs().max().item() <= 2.0 ** -7 * max(1.0, a.float().abs().max().item())
+
+
 # ------------------------------------------------------------------ full-size properties
 def test_config3_full_size_properties(device):
     """At B=2,H=16,S=4096,D=128 the oracle is too slow for the whole tensor; check it on a few

@@ -176,6 +176,18 @@ int tri_attn_bwd_dq(const TriAttnArgs* args) {
 }
 
 int tri_attn_bwd(const TriAttnArgs* args) {
+    // Where the dQ kernel can compute delta on the way (it loads the dO rows anyway), the pre-pass is
+    // dropped and dQ runs first: dK/dV reads the delta it stored.
+    {
+        KParams p;
+        int rc = make_params(args, 2 | 8, &p);
+        if (rc) return rc;
+        if (mfma_supported(kMfmaDq, args->dtype, p) && mfma_dq_fuses_delta(p)) {
+            rc = launch_mfma_dq(args->dtype, p, static_cast<hipStream_t>(args->stream), true);
+            if (rc) return rc;
+            return tri_attn_bwd_dkdv(args);
+        }
+    }
     int rc = tri_attn_bwd_delta(args);
     if (rc) return rc;
     rc = tri_attn_bwd_dkdv(args);

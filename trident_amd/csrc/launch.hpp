@@ -15,7 +15,10 @@ int launch_generic_any(int which, int dtype, const KParams& p, hipStream_t strea
 enum MfmaKernel { kMfmaFwd = 0, kMfmaDkdv = 1, kMfmaDq = 2 };
 bool mfma_supported(int which, int dtype, const KParams& p);
 int launch_mfma_fwd(int dtype, const KParams& p, hipStream_t stream);
-int launch_mfma_dq(int dtype, const KParams& p, hipStream_t stream);
+// with_delta: the dQ pass also computes and stores delta (only where mfma_dq_fuses_delta() says so; the
+// dK/dV pass must then follow it)
+int launch_mfma_dq(int dtype, const KParams& p, hipStream_t stream, bool with_delta = false);
+bool mfma_dq_fuses_delta(const KParams& p);
 int launch_mfma_dkdv(int dtype, const KParams& p, hipStream_t stream);
 int launch_delta(int dtype, const KParams& p, hipStream_t stream);
 

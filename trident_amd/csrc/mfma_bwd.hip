@@ -247,7 +247,10 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
 // workgroup barrier after each; waves 4-7 run one phase behind waves 0-3. Tile loads are issued at
 // the top of the vector phase (two tiles ahead in waves 0-3, three in waves 4-7, which start their
 // phase later) and awaited before its barrier.
-template <typename T, int D, bool CAUSAL, bool DROPOUT>
+// With DELTA the kernel also computes delta = rowsum(dO * O) of its rows (instead of reading it) and stores
+// it for the dK/dV pass, which then has to run after this one: the separate pre-pass over O and dO
+// (trident/kernel/softmax.py:180-238) disappears into the prologue that loads the dO rows anyway.
+template <typename T, int D, bool CAUSAL, bool DROPOUT, bool DELTA>
 __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p) {
     using Tile = SwzTile<D>;
     constexpr int NW = 8;
@@ -288,9 +291,16 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
         qf[kk] = *reinterpret_cast<const u32x4*>(qrowp + (2 * kk + h) * 16);
         gf[kk] = *reinterpret_cast<const u32x4*>(gorowp + (2 * kk + h) * 16);
     }
+    u32x4 of[DELTA ? KK : 1];
+    if constexpr (DELTA) {
+        const char* orowp = static_cast<const char*>(p.o) + (b * p.os[0] + hd * p.os[1] + static_cast<int64_t>(qrow) * p.os[2]) * 2;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) of[kk] = *reinterpret_cast<const u32x4*>(orowp + (2 * kk + h) * 16);
+    }
     float lse = p.lse[static_cast<int64_t>(bh) * p.S + qrow];
     if (lse == -INFINITY) lse = INFINITY;  // fully masked row: every probability is 0
-    const float dlt = p.delta[static_cast<int64_t>(bh) * p.S + qrow];
+    float dlt = 0.f;
+    if constexpr (!DELTA) dlt = p.delta[static_cast<int64_t>(bh) * p.S + qrow];
     const float c = p.scale_log2;
 
     f32x16 acc[DB];
@@ -327,7 +337,21 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
         settle(gf[kk]);
     }
     settle(lse);
-    settle(dlt);
+    if constexpr (DELTA) {
+        // this lane holds half of its row (the other half is in lane ^ 32)
+        float part = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                part = fmaf(Mma<T>::lo(of[kk][i]), Mma<T>::lo(gf[kk][i]), part);
+                part = fmaf(Mma<T>::hi(of[kk][i]), Mma<T>::hi(gf[kk][i]), part);
+            }
+        dlt = sum_xor32(part);
+        if (h == 0) p.delta[static_cast<int64_t>(bh) * p.S + qrow] = dlt;
+    } else {
+        settle(dlt);
+    }
 
     const int row_off0 = Tile::off(l32, h);
     const int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
@@ -1100,23 +1124,32 @@ int launch_dq_waves(const KParams& p, hipStream_t stream) {
     return static_cast<int>(hipGetLastError());
 }
 
+// whether the phased dQ kernel serves this problem (no mask, 256-row workgroups; with dropout at D = 128 it
+// would not fit its registers)
+template <int D, int MASK>
+bool dq_is_phased(const KParams& p) {
+    return MASK == kNoMask && p.S % 256 == 0 && (D == 64 || p.thr8 <= 0);
+}
+
 template <typename T, int D, bool CAUSAL, int MASK>
-int launch_dq_dropout(const KParams& p, hipStream_t stream) {
-    // 8 waves (256 query rows) when the sequence allows it, else 4 waves (128 rows)
+int launch_dq_dropout(const KParams& p, hipStream_t stream, bool with_delta) {
     if constexpr (MASK == kNoMask) {
-        // the phased kernel (with dropout at D = 128 it would not fit its registers)
-        if (p.S % 256 == 0 && (D == 64 || p.thr8 <= 0)) {
+        if (dq_is_phased<D, MASK>(p)) {
             const dim3 grid(p.B * p.H * (p.S / 256)), block(512);
             if constexpr (D == 64) {
                 if (p.thr8 > 0) {
-                    hipLaunchKernelGGL((mfma_dq_phased_kernel<T, D, CAUSAL, true>), grid, block, 0, stream, p);
+                    if (with_delta) hipLaunchKernelGGL((mfma_dq_phased_kernel<T, D, CAUSAL, true, true>), grid, block, 0, stream, p);
+                    else hipLaunchKernelGGL((mfma_dq_phased_kernel<T, D, CAUSAL, true, false>), grid, block, 0, stream, p);
                     return static_cast<int>(hipGetLastError());
                 }
             }
-            hipLaunchKernelGGL((mfma_dq_phased_kernel<T, D, CAUSAL, false>), grid, block, 0, stream, p);
+            if (with_delta) hipLaunchKernelGGL((mfma_dq_phased_kernel<T, D, CAUSAL, false, true>), grid, block, 0, stream, p);
+            else hipLaunchKernelGGL((mfma_dq_phased_kernel<T, D, CAUSAL, false, false>), grid, block, 0, stream, p);
             return static_cast<int>(hipGetLastError());
         }
     }
+    if (with_delta) return TRI_ATTN_ESHAPE;  // (callers ask dq_fuses_delta first)
+    // 8 waves (256 query rows) when the sequence allows it, else 4 waves (128 rows)
     if (p.S % 256 == 0) return launch_dq_waves<T, D, 8, CAUSAL, MASK>(p, stream);
     return launch_dq_waves<T, D, 4, CAUSAL, MASK>(p, stream);
 }
@@ -1147,35 +1180,37 @@ int launch_dkdv_dropout(const KParams& p, hipStream_t stream) {
 }
 
 template <int WHICH, typename T, int D, bool CAUSAL, int MASK>
-int launch_bwd_dropout(const KParams& p, hipStream_t stream) {
+int launch_bwd_dropout(const KParams& p, hipStream_t stream, bool with_delta) {
     if constexpr (WHICH == kMfmaDq) {
-        return launch_dq_dropout<T, D, CAUSAL, MASK>(p, stream);
+        return launch_dq_dropout<T, D, CAUSAL, MASK>(p, stream, with_delta);
     } else {
         return launch_dkdv_dropout<T, D, CAUSAL, MASK>(p, stream);
     }
 }
 
 template <int WHICH, typename T, int D>
-int launch_bwd_variant(int dtype, const KParams& p, hipStream_t stream) {
-    if (p.causal) return launch_bwd_dropout<WHICH, T, D, true, kNoMask>(p, stream);
-    if (p.mask == nullptr) return launch_bwd_dropout<WHICH, T, D, false, kNoMask>(p, stream);
-    if (p.mask_dtype == TRI_ATTN_F32) return launch_bwd_dropout<WHICH, T, D, false, kMaskF32>(p, stream);
-    if (p.mask_dtype == dtype) return launch_bwd_dropout<WHICH, T, D, false, kMaskT>(p, stream);
+int launch_bwd_variant(int dtype, const KParams& p, hipStream_t stream, bool with_delta) {
+    if (p.causal) return launch_bwd_dropout<WHICH, T, D, true, kNoMask>(p, stream, with_delta);
+    if (p.mask == nullptr) return launch_bwd_dropout<WHICH, T, D, false, kNoMask>(p, stream, with_delta);
+    if (p.mask_dtype == TRI_ATTN_F32) return launch_bwd_dropout<WHICH, T, D, false, kMaskF32>(p, stream, with_delta);
+    if (p.mask_dtype == dtype) return launch_bwd_dropout<WHICH, T, D, false, kMaskT>(p, stream, with_delta);
     return TRI_ATTN_EDTYPE;
 }
 
 template <int WHICH>
-int launch_bwd(int dtype, const KParams& p, hipStream_t stream) {
+int launch_bwd(int dtype, const KParams& p, hipStream_t stream, bool with_delta) {
     if (dtype == TRI_ATTN_BF16)
-        return p.D == 128 ? launch_bwd_variant<WHICH, bf16_t, 128>(dtype, p, stream)
-                          : launch_bwd_variant<WHICH, bf16_t, 64>(dtype, p, stream);
-    return p.D == 128 ? launch_bwd_variant<WHICH, f16_t, 128>(dtype, p, stream)
-                      : launch_bwd_variant<WHICH, f16_t, 64>(dtype, p, stream);
+        return p.D == 128 ? launch_bwd_variant<WHICH, bf16_t, 128>(dtype, p, stream, with_delta)
+                          : launch_bwd_variant<WHICH, bf16_t, 64>(dtype, p, stream, with_delta);
+    return p.D == 128 ? launch_bwd_variant<WHICH, f16_t, 128>(dtype, p, stream, with_delta)
+                      : launch_bwd_variant<WHICH, f16_t, 64>(dtype, p, stream, with_delta);
 }
 
 }  // namespace
 
-int launch_mfma_dq(int dtype, const KParams& p, hipStream_t stream) { return launch_bwd<kMfmaDq>(dtype, p, stream); }
-int launch_mfma_dkdv(int dtype, const KParams& p, hipStream_t stream) { return launch_bwd<kMfmaDkdv>(dtype, p, stream); }
+int launch_mfma_dq(int dtype, const KParams& p, hipStream_t stream, bool with_delta) {
+    return launch_bwd<kMfmaDq>(dtype, p, stream, with_delta);
+}
+int launch_mfma_dkdv(int dtype, const KParams& p, hipStream_t stream) { return launch_bwd<kMfmaDkdv>(dtype, p, stream, false); }
 
 }  // namespace tri

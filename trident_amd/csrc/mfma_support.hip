@@ -80,6 +80,13 @@ bool mfma_supported(int which, int dtype, const KParams& p) {
     }
 }
 
+// The phased dQ kernel (no mask, 256-row workgroups, no dropout at D = 128) can compute delta itself.
+bool mfma_dq_fuses_delta(const KParams& p) {
+    if (p.mask != nullptr || p.S % 256 != 0) return false;
+    if (!(p.D == 64 || p.thr8 <= 0)) return false;
+    return aligned16(p.o) && strides8(p.os);
+}
+
 int launch_delta(int dtype, const KParams& p, hipStream_t stream) {
     const bool vec = (dtype == TRI_ATTN_F16 || dtype == TRI_ATTN_BF16) && (p.D == 64 || p.D == 128) &&
                      aligned16(p.o) && aligned16(p.d_o) && strides8(p.os) && strides8(p.dos) &&

@@ -200,13 +200,11 @@ class Attention(torch.autograd.Function):
         if grad_mask_full is not None:
             _fill(args, "dmask", grad_mask_full, "dmask_stride")
 
-        util.push_trace("kernel.Softmax.backward_delta")
-        _lib.check(lib.tri_attn_bwd_delta(ctypes.byref(args)))
-        util.pop_trace()
-
+        # one call for the three backward launches (trident/operation/attention.py:161-199 launches the
+        # delta pre-pass and the backward kernel): the library orders them, and where the dQ kernel can
+        # compute delta on its way the pre-pass disappears into it
         util.push_trace("kernel.Attention.backward")
-        _lib.check(lib.tri_attn_bwd_dkdv(ctypes.byref(args)))
-        _lib.check(lib.tri_attn_bwd_dq(ctypes.byref(args)))
+        _lib.check(lib.tri_attn_bwd(ctypes.byref(args)))
         util.pop_trace()
 
         grad_mask = None
