@@ -298,6 +298,16 @@ def test_lengths_that_are_not_powers_of_two(dtype, S, D, variant, device):
     _abi_case(device, dtype, S, D, variant, 300 + S + D)
 
 
+# ------------------------------------------------------------------ tile counts of the phased kernels
+@pytest.mark.parametrize("variant", ["plain", "causal", "causal+dropout"])
+@pytest.mark.parametrize("S,D", [(256, 128), (768, 128), (1280, 128), (768, 64), (1024, 64)])
+def test_phased_kernels_over_tile_counts(S, D, variant, device):
+    """Multiples of 256 that are not powers of two included (the operator API cannot pass those): 4 to 20
+    streamed tiles, so the prologue, the steady state and the drain of the load pipeline of the forward
+    and dQ kernels, and the waves that stop early under the causal mask, are all exercised."""
+    _abi_case(device, torch.bfloat16 if D == 128 else torch.float16, S, D, variant, 500 + S + D)
+
+
 # ------------------------------------------------------------------ the combined backward entry point
 @pytest.mark.parametrize("S,D,causal,p", [(512, 128, True, 0.0), (256, 64, False, 0.0), (512, 64, True, 0.25),
                                           (256, 128, True, 0.25), (384, 128, True, 0.0)])
