@@ -1115,6 +1115,321 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
     }
 }
 
+// ------------------------------------------------------------------ dK, dV (paired waves, phased; no mask)
+// The pairing of the kernel above (waves w and w+4 share key block w%4, each accumulates half of the
+// head dimension) with the phase structure of the forward kernel. Q and dO stream as 32-row blocks
+// (plus their lse and delta) through a ring of 7 slots; even blocks are scored by member 0, odd
+// blocks by member 1, and both members accumulate every block. A member alternates
+//   vector phase:  P and dS of its block from S and dP (softmax backward), published in its LDS slot;
+//                  the partner's latest block is fetched from the partner's slot;
+//   matrix phase:  dV^T, dK^T += the partner's latest block and its own (16 MFMAs), then S and dP of
+//                  its next block (16 MFMAs), through one ring of LDS fragments;
+// with a workgroup barrier after each phase, member 1 one phase behind member 0: a SIMD always has one
+// wave on the matrix pipe and one on the vector ALU. Block r is first read in phase r-1 and last in
+// phase r+2; in phase ph every wave issues its share of block ph+4 and, before the barrier, waits for
+// its share of block ph+2.
+template <typename T, int D, bool CAUSAL, bool DROPOUT>
+__global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams p) {
+    using Tile = SwzTile<D>;
+    constexpr int NW = 8;
+    constexpr int kKeys = 128;
+    constexpr int kBR = 32;                                  // rows per streamed block
+    constexpr int kSlots = 7;
+    constexpr int kHalfBytes = kBR * Tile::kRowBytes;        // one operand of a block
+    constexpr int kSlotBytes = 2 * kHalfBytes + 512;         // Q rows, dO rows, lse, delta (256 B each)
+    constexpr int kXchBytes = NW * 4096;                     // per wave: P[2], dS[2] fragments
+    constexpr int KK = D / 16;
+    constexpr int DB = D / 32;
+    constexpr int DH = DB / 2;                               // column blocks a pair member accumulates
+    constexpr int kLoads = 3;                                // loads per wave and block
+    static_assert(kHalfBytes == NW * 1024, "one Q load and one dO load per wave and block");
+    constexpr int kAccSteps = 4 * DH;                        // MFMAs that add one block
+    constexpr int kSteps = 2 * kAccSteps + 2 * KK;           // matrix phase
+    constexpr int kRing = 4;
+    __shared__ __attribute__((aligned(1024))) char smem[kSlots * kSlotBytes + kXchBytes];
+    char* xch = smem + kSlots * kSlotBytes;
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int kb = wave & 3, member = wave >> 2;
+    const int lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+    int bh, kt;
+    map_block(blockIdx.x, p.B * p.H, p.S / kKeys, CAUSAL ? kHeavyFirst : kUniformTiles, &bh, &kt);
+    const int b = bh / p.H, hd = bh % p.H;
+    const int k0 = kt * kKeys;
+    const int wkey0 = k0 + 32 * kb;
+    const int key = wkey0 + l32;
+
+    const char* kbase = static_cast<const char*>(p.k) + (b * p.ks[0] + hd * p.ks[1]) * 2;
+    const char* vbase = static_cast<const char*>(p.v) + (b * p.vs[0] + hd * p.vs[1]) * 2;
+    const char* qbase = static_cast<const char*>(p.q) + (b * p.qs[0] + hd * p.qs[1]) * 2;
+    const char* gbase = static_cast<const char*>(p.d_o) + (b * p.dos[0] + hd * p.dos[1]) * 2;
+    const int64_t qrow_bytes = p.qs[2] * 2, grow_bytes = p.dos[2] * 2;
+    const float* lse_base = p.lse + static_cast<int64_t>(bh) * p.S;
+    const float* delta_base = p.delta + static_cast<int64_t>(bh) * p.S;
+    const float c = p.scale_log2;
+
+    f32x16 dk[DH], dv[DH];
+#pragma unroll
+    for (int d = 0; d < DH; ++d) {
+        dk[d] = zero16();
+        dv[d] = zero16();
+    }
+
+    const int row_first = CAUSAL ? k0 : 0;          // first streamed row (block 0)
+    const int n_blocks = (p.S - row_first) / kBR;   // >= 4, even
+    const uint32_t qoff = static_cast<uint32_t>(Tile::src_off(wave, lane, qrow_bytes));
+    const uint32_t goff = static_cast<uint32_t>(Tile::src_off(wave, lane, grow_bytes));
+    auto slot_of = [&](int r) { return smem + ((r + kSlots) % kSlots) * kSlotBytes; };
+    auto issue_block = [&](int r) {  // this wave's share of block r, if it exists
+        if (r < n_blocks) {
+            char* slot = slot_of(r);
+            const int64_t row = row_first + static_cast<int64_t>(r) * kBR;
+            lds_direct_load16(qbase + row * qrow_bytes, qoff, slot + wave * 1024);
+            lds_direct_load16(gbase + row * grow_bytes, goff, slot + kHalfBytes + wave * 1024);
+            // even waves fetch the 32 lse values, odd waves the 32 delta values (lanes 32-63 repeat them)
+            if (wave & 1) lds_direct_load4(delta_base + row, (lane & 31) * 4, slot + 2 * kHalfBytes + 256);
+            else lds_direct_load4(lse_base + row, (lane & 31) * 4, slot + 2 * kHalfBytes);
+        }
+    };
+    // before the barrier that ends phase ph: block ph+2 has landed, blocks ph+3 and ph+4 may be in flight
+    auto wait_blocks = [&](int ph) {
+        const int young = (ph + 3 < n_blocks ? 1 : 0) + (ph + 4 < n_blocks ? 1 : 0);
+        if (young == 2) TRI_WAIT_VMCNT(2 * kLoads);
+        else if (young == 1) TRI_WAIT_VMCNT(kLoads);
+        else TRI_WAIT_VMCNT(0);
+    };
+
+    // The K and V rows of the workgroup (128 keys = two 64-row tiles each) arrive through LDS too (lanes
+    // own keys, so direct loads would touch 32 cache lines per instruction); they land behind the first
+    // four ring slots, which take blocks 0-3 meanwhile.
+    char* kv_lds = smem + 4 * kSlotBytes;
+    static_assert(3 * kSlotBytes + kXchBytes >= 4 * Tile::kBytes, "K and V must fit behind the first four slots");
+    constexpr int kKvLoads = 4 * Tile::kBlocks / NW;
+    {
+        const int64_t krow_bytes = p.ks[2] * 2, vrow_bytes = p.vs[2] * 2;
+#pragma unroll
+        for (int i = 0; i < kKvLoads; ++i) {
+            const int blk = wave * kKvLoads + i;           // 0 .. 4*kBlocks-1: K tile 0, K tile 1, V tile 0, V tile 1
+            const int tile = blk / Tile::kBlocks, b16 = blk % Tile::kBlocks;
+            const bool is_v = tile >= 2;
+            const int64_t rb = is_v ? vrow_bytes : krow_bytes;
+            const char* src = (is_v ? vbase : kbase) + (k0 + 64 * (tile & 1)) * rb;
+            lds_direct_load16(src, static_cast<uint32_t>(Tile::src_off(b16, lane, rb)), kv_lds + blk * 1024);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) issue_block(r);
+
+    const int row_off0 = Tile::off(l32, h);
+    const int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
+    TRI_WAIT_VMCNT(4 * kLoads);  // K and V have landed
+    lds_barrier();
+    u32x4 kf[KK], vf[KK];
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+        const int off = (row_off0 ^ (kk << 5)) + 32 * (kb & 1) * Tile::kRowBytes;
+        kf[kk] = lds_read16(kv_lds + (kb >> 1) * Tile::kBytes, off);
+        vf[kk] = lds_read16(kv_lds + (2 + (kb >> 1)) * Tile::kBytes, off);
+    }
+    lds_barrier();  // every wave has its fragments: the region is free for the exchange slots and later blocks
+    char* my_xch = xch + wave * 4096 + lane * 16;
+    const char* peer_xch = xch + (wave ^ 4) * 4096 + lane * 16;
+    u32x4 cur_p[2], cur_s[2];   // P and dS of this member's current block
+    u32x4 par_p[2], par_s[2];   // the partner's latest block
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+        cur_p[g] = cur_s[g] = par_p[g] = par_s[g] = u32x4{0, 0, 0, 0};
+        *reinterpret_cast<u32x4*>(my_xch + g * 1024) = cur_p[g];
+        *reinterpret_cast<u32x4*>(my_xch + (2 + g) * 1024) = cur_s[g];
+    }
+    TRI_WAIT_VMCNT(2 * kLoads);  // blocks 0 and 1 have landed
+    lds_barrier();
+
+    // whether this pair has anything in block r (under the causal mask: rows at or below its first key)
+    auto block_on = [&](int r) { return r >= 0 && r < n_blocks && (!CAUSAL || r >= kb); };
+    auto clamp_block = [&](int r) { return r < 0 ? 0 : (r >= n_blocks ? n_blocks - 1 : r); };
+
+    f32x16 sc_s, sc_dp;  // S and dP of this member's next block
+    u32x4 ring[kRing];
+    // fragment n of a matrix phase that adds blocks ra and rb and scores block rs
+    auto frag = [&](int ra, int rb, int rs, int n) {
+        if (n < 2 * kAccSteps) {
+            const char* slot = slot_of(n < kAccSteps ? ra : rb);
+            const int m = n % kAccSteps;
+            const int d = m % DH, which = (m / DH) % 2, g = m / (2 * DH);
+            const int db = DH * member + d;
+            return Tile::tr_frag(slot + (which ? 0 : kHalfBytes), tr_off0 ^ (db << 6), tr_off1 ^ (db << 6), g);
+        }
+        const int m = n - 2 * kAccSteps;
+        return lds_read16(slot_of(rs) + (m < KK ? 0 : kHalfBytes), row_off0 ^ ((m % KK) << 5));
+    };
+    auto matrix_phase = [&](auto with_acc, int ra, int rb, int rs) {
+        constexpr int first = decltype(with_acc)::value ? 0 : 2 * kAccSteps;
+        f32x16 s = zero16(), dp = zero16();
+#pragma unroll
+        for (int n = first; n < kSteps; ++n) {
+            const int slot = (n - first) % kRing;
+            if (n < 2 * kAccSteps) {
+                const int m = n % kAccSteps;
+                const int d = m % DH, which = (m / DH) % 2, g = m / (2 * DH);
+                const bool own = n >= kAccSteps;
+                if (which == 0) dv[d] = Mma<T>::run(ring[slot], own ? cur_p[g] : par_p[g], dv[d]);
+                else dk[d] = Mma<T>::run(ring[slot], own ? cur_s[g] : par_s[g], dk[d]);
+            } else {
+                const int m = n - 2 * kAccSteps;
+                if (m < KK) s = Mma<T>::run(ring[slot], kf[m], s);
+                else dp = Mma<T>::run(ring[slot], vf[m - KK], dp);
+            }
+            if (n + kRing < kSteps) ring[slot] = frag(ra, rb, rs, n + kRing);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        sc_s = s;
+        sc_dp = dp;
+    };
+    using Yes = std::integral_constant<bool, true>;
+    using No = std::integral_constant<bool, false>;
+
+    // vector phase for block r (this member's): P and dS from sc_s, sc_dp
+    auto vector_phase = [&](int r) {
+        if (block_on(r)) {
+            const char* slot = slot_of(r);
+            const float* sLse = reinterpret_cast<const float*>(slot + 2 * kHalfBytes);
+            const float* sDelta = sLse + 64;
+            const int rb = row_first + r * kBR;
+            const bool diag = CAUSAL && r == kb;
+            const f32x16 s = sc_s, dp = sc_dp;
+            f32x4 lse4[4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) lse4[g] = *reinterpret_cast<const f32x4*>(sLse + 8 * g + 4 * h);
+            Philox4 mine;  // the block of rows rb + 8 (lane % 4) + 4 h .. +3: this lane's share of the quad's four
+            if constexpr (DROPOUT) mine = dropout_block(p, bh, (rb + 8 * (lane & 3) + 4 * h) >> 2, key >> 2);
+#pragma unroll
+            for (int gg = 0; gg < 2; ++gg) {  // eight rows at a time, packed as soon as they are done
+                float pr[8], ds[8];
+                f32x4 dlt4[2];
+#pragma unroll
+                for (int g2 = 0; g2 < 2; ++g2) dlt4[g2] = *reinterpret_cast<const f32x4*>(sDelta + 8 * (2 * gg + g2) + 4 * h);
+#pragma unroll
+                for (int g2 = 0; g2 < 2; ++g2) {
+                    const int g = 2 * gg + g2;
+                    const f32x4 l4 = lse4[g];
+                    const f32x4 d4 = dlt4[g2];
+                    uint32_t dw[4];
+                    if constexpr (DROPOUT) {
+                        const Philox4 rr = quad_bcast_from(g, mine);  // lane g of the quad generated rows rb + 8 g + 4 h .. +3
+#pragma unroll
+                        for (int bb = 0; bb < 4; ++bb) dw[bb] = (rr.w[bb] >> (8 * (key & 3))) & 0xffu;
+                    }
+#pragma unroll
+                    for (int bb = 0; bb < 4; ++bb) {
+                        const int i = 4 * g + bb;
+                        float pv = fast_exp2(fmaf(s[i], c, -l4[bb]));
+                        if (diag) pv = key <= rb + c_row(i, h) ? pv : 0.f;
+                        float dpv = dp[i];
+                        if constexpr (DROPOUT) {
+                            const bool keep = static_cast<int>(dw[bb]) >= p.thr8;
+                            dpv = keep ? dpv * p.zscale : 0.f;
+                            pr[4 * g2 + bb] = keep ? pv * p.zscale : 0.f;
+                        } else {
+                            pr[4 * g2 + bb] = pv;
+                        }
+                        ds[4 * g2 + bb] = pv * (dpv - d4[bb]);
+                    }
+                }
+                cur_p[gg] = pack8<T>(pr);
+                cur_s[gg] = pack8<T>(ds);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+#pragma unroll
+            for (int g = 0; g < 2; ++g) cur_p[g] = cur_s[g] = u32x4{0, 0, 0, 0};
+        }
+    };
+    // the second half of a vector phase in global phase ph, for a member whose block is r: publish, fetch
+    // the partner's block r-1, request the first fragments of the matrix phase, meet the barrier
+    auto close_vector_phase = [&](int ph, int r) {
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            *reinterpret_cast<u32x4*>(my_xch + g * 1024) = cur_p[g];
+            *reinterpret_cast<u32x4*>(my_xch + (2 + g) * 1024) = cur_s[g];
+        }
+        issue_block(ph + 4);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // published before the barrier
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            par_p[g] = *reinterpret_cast<const u32x4*>(peer_xch + g * 1024);
+            par_s[g] = *reinterpret_cast<const u32x4*>(peer_xch + (2 + g) * 1024);
+        }
+        const int ra = clamp_block(r - 1), rb = clamp_block(r);
+#pragma unroll
+        for (int n = 0; n < kRing; ++n) ring[n] = frag(ra, rb, r + 2, n);
+        wait_blocks(ph);
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_barrier" ::: "memory");  // (the reads above stay in flight)
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto run_matrix_phase = [&](int ph, int r) {
+        __builtin_amdgcn_s_setprio(2);
+        matrix_phase(Yes{}, clamp_block(r - 1), clamp_block(r), r + 2);
+        __builtin_amdgcn_s_setprio(0);
+        issue_block(ph + 4);
+        wait_blocks(ph);
+        __builtin_amdgcn_sched_barrier(0);
+        lds_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto idle_phase = [&](int ph) {
+        issue_block(ph + 4);
+        wait_blocks(ph);
+        lds_barrier();
+    };
+
+    // before phase 0: S and dP of each member's first block (member 0: block 0, member 1: block 1)
+    {
+#pragma unroll
+        for (int n = 0; n < kRing; ++n) ring[n] = frag(0, 0, member, 2 * kAccSteps + n);
+        __builtin_amdgcn_sched_barrier(0);
+        matrix_phase(No{}, 0, 0, member);
+        lds_barrier();
+    }
+    const int n_iter = n_blocks / 2;
+    if (member == 0) {
+#pragma unroll 1
+        for (int t = 0; t <= n_iter; ++t) {   // the last round only adds member 1's last block
+            const int r = 2 * t;
+            vector_phase(r);
+            close_vector_phase(2 * t, r);
+            run_matrix_phase(2 * t + 1, r);
+        }
+    } else {
+        idle_phase(0);
+#pragma unroll 1
+        for (int t = 0; t < n_iter; ++t) {
+            const int r = 2 * t + 1;
+            vector_phase(r);
+            close_vector_phase(2 * t + 1, r);
+            run_matrix_phase(2 * t + 2, r);
+        }
+        idle_phase(2 * n_iter + 1);
+    }
+
+    // every wave is out of the loop: the ring can serve as the waves' private transposition patches
+    lds_barrier();
+    {
+        using Store = RowBlockStore<T, DH>;
+        static_assert(NW * Store::kPatchBytes <= kSlots * kSlotBytes, "patches must fit into the ring");
+        char* patch = smem + wave * Store::kPatchBytes;
+        const int64_t row = wkey0;  // first key of this pair; this member writes columns 32*DH*member ..
+        char* dk0 = static_cast<char*>(p.dk) + (b * p.dks[0] + hd * p.dks[1] + row * p.dks[2] + 32 * DH * member) * 2;
+        char* dv0 = static_cast<char*>(p.dv) + (b * p.dvs[0] + hd * p.dvs[1] + row * p.dvs[2] + 32 * DH * member) * 2;
+        const float sc = p.scale;
+        Store::run(dk, [sc](float x) { return x * sc; }, patch, dk0, p.dks[2] * 2, lane);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // patch read before it is rewritten
+        Store::run(dv, [](float x) { return x; }, patch, dv0, p.dvs[2] * 2, lane);
+    }
+}
+
 // ---------------------------------------------------------------------------------- launch
 template <typename T, int D, int NW, bool CAUSAL, int MASK>
 int launch_dq_waves(const KParams& p, hipStream_t stream) {
@@ -1173,6 +1488,12 @@ int launch_dkdv_dropout(const KParams& p, hipStream_t stream) {
         // D = 128: K, V and both gradient accumulators of a 32-key block take 192 registers, too many
         // for two waves per SIMD, so two waves are paired on each key block of a 128-key workgroup
         const dim3 grid(p.B * p.H * (p.S / kBM)), block(512);
+        if constexpr (MASK == kNoMask) {
+            if (p.thr8 <= 0) {
+                hipLaunchKernelGGL((mfma_dkdv_phased_kernel<T, D, CAUSAL, false>), grid, block, 0, stream, p);
+                return static_cast<int>(hipGetLastError());
+            }
+        }
         if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dkdv_pair_kernel<T, D, CAUSAL, MASK, true>), grid, block, 0, stream, p);
         else hipLaunchKernelGGL((mfma_dkdv_pair_kernel<T, D, CAUSAL, MASK, false>), grid, block, 0, stream, p);
         return static_cast<int>(hipGetLastError());
