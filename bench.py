@@ -70,16 +70,25 @@ class Path:
         operation._fill(args, "delta", self.delta)
         self.args = args
         ref = ctypes.byref(args)
+        # A step is the launch sequence of the operator (tri_attn_fwd, then what tri_attn_bwd launches): where
+        # the fused dQ + delta kernel applies, dQ (with delta) and dK/dV; otherwise delta, dK/dV, dQ.
         self.kernels = [("fwd", lambda: self.check(self.lib.tri_attn_fwd(ref)))]
-        # a step: what the operator launches (forward, then the whole backward in one call)
-        self.step_calls = [lambda: self.check(self.lib.tri_attn_fwd(ref))]
         if w.backward:
-            self.kernels += [
-                ("bwd_delta", lambda: self.check(self.lib.tri_attn_bwd_delta(ref))),
-                ("bwd_dkdv", lambda: self.check(self.lib.tri_attn_bwd_dkdv(ref))),
-                ("bwd_dq", lambda: self.check(self.lib.tri_attn_bwd_dq(ref))),
-            ]
-            self.step_calls.append(lambda: self.check(self.lib.tri_attn_bwd(ref)))
+            self.check(self.lib.tri_attn_fwd(ref))
+            rc = self.lib.tri_attn_bwd_dq_delta(ref)
+            if rc == 0:
+                self.kernels += [
+                    ("bwd_dq", lambda: self.check(self.lib.tri_attn_bwd_dq_delta(ref))),
+                    ("bwd_dkdv", lambda: self.check(self.lib.tri_attn_bwd_dkdv(ref))),
+                ]
+            elif rc == _lib.ENOFUSE:
+                self.kernels += [
+                    ("bwd_delta", lambda: self.check(self.lib.tri_attn_bwd_delta(ref))),
+                    ("bwd_dkdv", lambda: self.check(self.lib.tri_attn_bwd_dkdv(ref))),
+                    ("bwd_dq", lambda: self.check(self.lib.tri_attn_bwd_dq(ref))),
+                ]
+            else:
+                self.check(rc)
 
     def algorithmic_flops(self, kernel):
         """Flops credited per launch: forward 4 B H S^2 D; of the 10 B H S^2 D of the backward,
@@ -97,32 +106,24 @@ class Path:
 
 
 def run_steps(path, steps, warmup):
-    """Returns (ms per step by wall clock, {kernel: avg ms} from HIP events on the launch stream).
-
-    The wall clock is taken over `steps` steps as the operator launches them (forward, then the backward
-    through tri_attn_bwd, which folds the delta pre-pass into the dQ kernel where it can). The per-kernel
-    figures come from a second, separately launched series of the individual entry points."""
+    """Returns (ms per step by wall clock, {kernel: avg ms} from HIP events on the launch stream)."""
     import torch
 
     for _ in range(warmup):
-        for fn in path.step_calls:
+        for _, fn in path.kernels:
             fn()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        for fn in path.step_calls:
-            fn()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-
     n = len(path.kernels)
     events = [[torch.cuda.Event(enable_timing=True) for _ in range(n + 1)] for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
     for s in range(steps):
         events[s][0].record()
         for i, (_, fn) in enumerate(path.kernels):
             fn()
             events[s][i + 1].record()
     torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     per_kernel = {}
     for i, (name, _) in enumerate(path.kernels):
         per_kernel[name] = sum(events[s][i].elapsed_time(events[s][i + 1]) for s in range(steps)) / steps

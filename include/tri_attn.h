@@ -58,7 +58,8 @@ enum {
     TRI_ATTN_EMASKCAUSAL = -5,/* both mask and is_causal set */
     TRI_ATTN_EDROPOUT = -6,   /* dropout_p outside [0,1] */
     TRI_ATTN_ESIZE = -7,      /* struct_size does not match this ABI version */
-    TRI_ATTN_EALIGN = -8      /* a pointer or stride breaks the 16-byte alignment the kernels need */
+    TRI_ATTN_EALIGN = -8,     /* a pointer or stride breaks the 16-byte alignment the kernels need */
+    TRI_ATTN_ENOFUSE = -9     /* tri_attn_bwd_dq_delta only: no fused kernel serves this problem, nothing was launched */
 };
 
 typedef struct TriAttnArgs {
@@ -123,6 +124,14 @@ int tri_attn_bwd_dkdv(const TriAttnArgs* args);
  * (the reference accumulates into a zeroed dQ, trident/kernel/attention.py:321-323).
  * Reads q,k,v,d_o,lse,delta[,mask]; writes dq[, dmask]. */
 int tri_attn_bwd_dq(const TriAttnArgs* args);
+
+/* bwd_delta and bwd_dq in one launch, for the problems whose dQ kernel can compute delta from the dO
+ * rows it loads anyway (no mask, S a multiple of 256, fp16/bf16 with D in {64,128}, no dropout at
+ * D = 128): reads q,k,v,o,d_o,lse; writes delta and dq. tri_attn_bwd_dkdv, which reads delta, has to
+ * follow it. Returns TRI_ATTN_ENOFUSE without launching anything where it does not apply (then call
+ * tri_attn_bwd_delta, tri_attn_bwd_dkdv, tri_attn_bwd_dq). The reference has the two launches only
+ * (trident/operation/attention.py:161-199); tri_attn_bwd picks between the two sequences itself. */
+int tri_attn_bwd_dq_delta(const TriAttnArgs* args);
 
 /* The whole backward (trident/operation/attention.py:137-202): the results of bwd_delta, bwd_dkdv and
  * bwd_dq called in that order, written to delta, dk, dv, dq[, dmask]. The library may launch fewer

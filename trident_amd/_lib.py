@@ -4,6 +4,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtrident_attn.so")
+ENOFUSE = -9  # tri_attn_bwd_dq_delta: no fused kernel for this problem, nothing launched
 ABI_VERSION = 1
 
 _i64x4 = ctypes.c_int64 * 4
@@ -56,6 +57,7 @@ EXPORTS = (
     "tri_attn_bwd_delta",
     "tri_attn_bwd_dkdv",
     "tri_attn_bwd_dq",
+    "tri_attn_bwd_dq_delta",
     "tri_attn_bwd",
     "tri_attn_dropout_mask",
 )
@@ -78,7 +80,8 @@ def lib():
         cdll.tri_attn_version.restype = ctypes.c_int
         cdll.tri_attn_strerror.restype = ctypes.c_char_p
         cdll.tri_attn_strerror.argtypes = [ctypes.c_int]
-        for name in ("tri_attn_fwd", "tri_attn_bwd_delta", "tri_attn_bwd_dkdv", "tri_attn_bwd_dq", "tri_attn_bwd"):
+        for name in ("tri_attn_fwd", "tri_attn_bwd_delta", "tri_attn_bwd_dkdv", "tri_attn_bwd_dq",
+                     "tri_attn_bwd_dq_delta", "tri_attn_bwd"):
             fn = getattr(cdll, name)
             fn.restype = ctypes.c_int
             fn.argtypes = [ctypes.POINTER(TriAttnArgs)]

@@ -135,6 +135,7 @@ const char* tri_attn_strerror(int status) {
         case TRI_ATTN_EDROPOUT: return "dropout_p must lie in [0, 1]";
         case TRI_ATTN_ESIZE: return "TriAttnArgs.struct_size does not match this library";
         case TRI_ATTN_EALIGN: return "pointer or stride alignment not supported";
+        case TRI_ATTN_ENOFUSE: return "no fused dQ + delta kernel for this problem (nothing launched)";
         default: break;
     }
     if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
@@ -175,20 +176,21 @@ int tri_attn_bwd_dq(const TriAttnArgs* args) {
     return launch_generic_any(kGenericDq, args->dtype, p, st);
 }
 
+int tri_attn_bwd_dq_delta(const TriAttnArgs* args) {
+    KParams p;
+    int rc = make_params(args, 2 | 8, &p);
+    if (rc) return rc;
+    if (!(mfma_supported(kMfmaDq, args->dtype, p) && mfma_dq_fuses_delta(p))) return TRI_ATTN_ENOFUSE;
+    return launch_mfma_dq(args->dtype, p, static_cast<hipStream_t>(args->stream), true);
+}
+
 int tri_attn_bwd(const TriAttnArgs* args) {
     // Where the dQ kernel can compute delta on the way (it loads the dO rows anyway), the pre-pass is
     // dropped and dQ runs first: dK/dV reads the delta it stored.
-    {
-        KParams p;
-        int rc = make_params(args, 2 | 8, &p);
-        if (rc) return rc;
-        if (mfma_supported(kMfmaDq, args->dtype, p) && mfma_dq_fuses_delta(p)) {
-            rc = launch_mfma_dq(args->dtype, p, static_cast<hipStream_t>(args->stream), true);
-            if (rc) return rc;
-            return tri_attn_bwd_dkdv(args);
-        }
-    }
-    int rc = tri_attn_bwd_delta(args);
+    int rc = tri_attn_bwd_dq_delta(args);
+    if (rc == TRI_ATTN_OK) return tri_attn_bwd_dkdv(args);
+    if (rc != TRI_ATTN_ENOFUSE) return rc;
+    rc = tri_attn_bwd_delta(args);
     if (rc) return rc;
     rc = tri_attn_bwd_dkdv(args);
     if (rc) return rc;
