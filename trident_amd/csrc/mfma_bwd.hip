@@ -1250,7 +1250,10 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
     auto block_on = [&](int r) { return r >= 0 && r < n_blocks && (!CAUSAL || r >= kb); };
     auto clamp_block = [&](int r) { return r < 0 ? 0 : (r >= n_blocks ? n_blocks - 1 : r); };
 
-    f32x16 sc_s, sc_dp;  // S and dP of this member's next block
+    constexpr bool kFold = !DROPOUT;
+    constexpr float kFoldUnit = 256.f;  // the constant the split terms multiply (keeps f16 terms in range)
+    const float neg_inv_c = -1.f / c;
+    f32x16 sc_s, sc_dp;  // S and dP of this member's next block (S - lse / c and dP - delta when folded)
     u32x4 ring[kRing];
     // fragment n of a matrix phase that adds blocks ra and rb and scores block rs
     auto frag = [&](int ra, int rb, int rs, int n) {
@@ -1267,9 +1270,30 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
     auto matrix_phase = [&](auto with_acc, int ra, int rb, int rs) {
         constexpr int first = decltype(with_acc)::value ? 0 : 2 * kAccSteps;
         f32x16 s = zero16(), dp = zero16();
+        // Without dropout one more MFMA each puts -lse / c and -delta under S and dP (a row's value split
+        // into three 16-bit terms against a column of constants), so that the vector phase needs neither
+        // value: P = exp2(c S'), dS = P dP'. Each lane asks for its row's two values at the start.
+        constexpr int kReadStep = first;
+        float row_lse = 0.f, row_delta = 0.f;
 #pragma unroll
         for (int n = first; n < kSteps; ++n) {
             const int slot = (n - first) % kRing;
+            if constexpr (kFold) {
+                if (n == kReadStep) {
+                    const float* sLse = reinterpret_cast<const float*>(slot_of(rs) + 2 * kHalfBytes);
+                    row_lse = sLse[l32];
+                    row_delta = sLse[64 + l32];
+                }
+                if (n == 2 * kAccSteps) {
+                    const u32x4 zero4 = {0, 0, 0, 0};
+                    const u32x4 al = split3<T>(row_lse * neg_inv_c * (1.f / kFoldUnit));
+                    const u32x4 ad = split3<T>(row_delta * (-1.f / kFoldUnit));
+                    const uint32_t u2 = Mma<T>::pack2(kFoldUnit, kFoldUnit), u1 = Mma<T>::pack2(kFoldUnit, 0.f);
+                    const u32x4 units = h == 0 ? u32x4{u2, u1, 0, 0} : zero4;
+                    s = Mma<T>::run(h == 0 ? al : zero4, units, s);
+                    dp = Mma<T>::run(h == 0 ? ad : zero4, units, dp);
+                }
+            }
             if (n < 2 * kAccSteps) {
                 const int m = n % kAccSteps;
                 const int d = m % DH, which = (m / DH) % 2, g = m / (2 * DH);
@@ -1301,8 +1325,10 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
             const bool diag = CAUSAL && r == kb;
             const f32x16 s = sc_s, dp = sc_dp;
             f32x4 lse4[4];
+            if constexpr (!kFold) {
 #pragma unroll
-            for (int g = 0; g < 4; ++g) lse4[g] = *reinterpret_cast<const f32x4*>(sLse + 8 * g + 4 * h);
+                for (int g = 0; g < 4; ++g) lse4[g] = *reinterpret_cast<const f32x4*>(sLse + 8 * g + 4 * h);
+            }
             // a load instruction holds the wave until the memory pipeline takes it: with the uneven block
             // counts of a causal launch it costs least here, while the lse values are on their way (measured:
             // 3.6 % fewer cycles than at the end of the phase, where the even non-causal launch does 2 % better)
@@ -1314,7 +1340,9 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
                 float pr[8], ds[8];
                 f32x4 dlt4[2];
 #pragma unroll
-                for (int g2 = 0; g2 < 2; ++g2) dlt4[g2] = *reinterpret_cast<const f32x4*>(sDelta + 8 * (2 * gg + g2) + 4 * h);
+                for (int g2 = 0; g2 < 2; ++g2) {
+                    if constexpr (!kFold) dlt4[g2] = *reinterpret_cast<const f32x4*>(sDelta + 8 * (2 * gg + g2) + 4 * h);
+                }
 #pragma unroll
                 for (int g2 = 0; g2 < 2; ++g2) {
                     const int g = 2 * gg + g2;
@@ -1329,7 +1357,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
 #pragma unroll
                     for (int bb = 0; bb < 4; ++bb) {
                         const int i = 4 * g + bb;
-                        float pv = fast_exp2(fmaf(s[i], c, -l4[bb]));
+                        float pv = kFold ? fast_exp2(s[i] * c) : fast_exp2(fmaf(s[i], c, -l4[bb]));
                         if (diag) pv = key <= rb + c_row(i, h) ? pv : 0.f;
                         float dpv = dp[i];
                         if constexpr (DROPOUT) {
@@ -1339,7 +1367,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
                         } else {
                             pr[4 * g2 + bb] = pv;
                         }
-                        ds[4 * g2 + bb] = pv * (dpv - d4[bb]);
+                        ds[4 * g2 + bb] = kFold ? pv * dpv : pv * (dpv - d4[bb]);
                     }
                 }
                 cur_p[gg] = pack8<T>(pr);

@@ -79,6 +79,19 @@ __device__ __forceinline__ u32x4 pack8(const float* x) {
     return r;
 }
 
+// x as three 16-bit terms (K-slots 0-2 of an operand, the rest zero): their sum restores x to fp32 precision.
+template <typename T>
+__device__ __forceinline__ u32x4 split3(float x) {
+    const float a = static_cast<float>(static_cast<T>(x));
+    const float r1 = x - a;
+    const float b = static_cast<float>(static_cast<T>(r1));
+    u32x4 r;
+    r.x = Mma<T>::pack2(a, b);
+    r.y = Mma<T>::pack2(r1 - b, 0.f);
+    r.z = r.w = 0;
+    return r;
+}
+
 __device__ __forceinline__ f32x16 zero16() {
     f32x16 z;
 #pragma unroll
