@@ -1120,15 +1120,15 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
 // head dimension) with the phase structure of the forward kernel. Q and dO stream as 32-row blocks
 // (plus their lse and delta) through a ring of 7 slots; even blocks are scored by member 0, odd
 // blocks by member 1, and both members accumulate every block. A member alternates
-//   vector phase:  P and dS of its block from S and dP (softmax backward), published in its LDS slot;
+//   vector phase:  P and dS of its block from S' and dP' (softmax backward), published in its LDS slot;
 //                  the partner's latest block is fetched from the partner's slot;
-//   matrix phase:  dV^T, dK^T += the partner's latest block and its own (16 MFMAs), then S and dP of
-//                  its next block (16 MFMAs), through one ring of LDS fragments;
+//   matrix phase:  dV^T, dK^T += the partner's latest block and its own (16 MFMAs), then S' = S - lse / c
+//                  and dP' = dP - delta of its next block (18 MFMAs), through one ring of LDS fragments;
 // with a workgroup barrier after each phase, member 1 one phase behind member 0: a SIMD always has one
 // wave on the matrix pipe and one on the vector ALU. Block r is first read in phase r-1 and last in
 // phase r+2; in phase ph every wave issues its share of block ph+4 and, before the barrier, waits for
 // its share of block ph+2.
-template <typename T, int D, bool CAUSAL, bool DROPOUT>
+template <typename T, int D, bool CAUSAL>
 __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams p) {
     using Tile = SwzTile<D>;
     constexpr int NW = 8;
@@ -1181,16 +1181,26 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
     const uint32_t qoff = static_cast<uint32_t>(Tile::src_off(wave, lane, qrow_bytes));
     const uint32_t goff = static_cast<uint32_t>(Tile::src_off(wave, lane, grow_bytes));
     auto slot_of = [&](int r) { return smem + ((r + kSlots) % kSlots) * kSlotBytes; };
-    auto issue_block = [&](int r) {  // this wave's share of block r, if it exists
-        if (r < n_blocks) {
-            char* slot = slot_of(r);
-            const int64_t row = row_first + static_cast<int64_t>(r) * kBR;
-            lds_direct_load16(qbase + row * qrow_bytes, qoff, slot + wave * 1024);
-            lds_direct_load16(gbase + row * grow_bytes, goff, slot + kHalfBytes + wave * 1024);
-            // even waves fetch the 32 lse values, odd waves the 32 delta values (lanes 32-63 repeat them)
-            if (wave & 1) lds_direct_load4(delta_base + row, (lane & 31) * 4, slot + 2 * kHalfBytes + 256);
-            else lds_direct_load4(lse_base + row, (lane & 31) * 4, slot + 2 * kHalfBytes);
+    // Blocks are requested in order, one per phase (block ph + 4 in phase ph) after the first four: the
+    // source pointers and the ring slot advance with every call. Even waves fetch the 32 lse values of a
+    // block, odd waves its 32 delta values (lanes 32-63 repeat them).
+    int next_block = 0, next_slot = 0;
+    const char* next_q = qbase + row_first * qrow_bytes;
+    const char* next_g = gbase + row_first * grow_bytes;
+    const float* next_aux = ((wave & 1) ? delta_base : lse_base) + row_first;
+    const int aux_lds = 2 * kHalfBytes + ((wave & 1) ? 256 : 0);
+    auto issue_block = [&]() {  // this wave's share of the next block, if it exists
+        if (next_block < n_blocks) {
+            char* slot = smem + next_slot * kSlotBytes;
+            lds_direct_load16(next_q, qoff, slot + wave * 1024);
+            lds_direct_load16(next_g, goff, slot + kHalfBytes + wave * 1024);
+            lds_direct_load4(next_aux, (lane & 31) * 4, slot + aux_lds);
         }
+        ++next_block;
+        next_slot = next_slot == kSlots - 1 ? 0 : next_slot + 1;
+        next_q += kBR * qrow_bytes;
+        next_g += kBR * grow_bytes;
+        next_aux += kBR;
     };
     // before the barrier that ends phase ph: block ph+2 has landed, blocks ph+3 and ph+4 may be in flight
     auto wait_blocks = [&](int ph) {
@@ -1219,7 +1229,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
         }
     }
 #pragma unroll
-    for (int r = 0; r < 4; ++r) issue_block(r);
+    for (int r = 0; r < 4; ++r) issue_block();
 
     const int row_off0 = Tile::off(l32, h);
     const int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
@@ -1250,10 +1260,9 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
     auto block_on = [&](int r) { return r >= 0 && r < n_blocks && (!CAUSAL || r >= kb); };
     auto clamp_block = [&](int r) { return r < 0 ? 0 : (r >= n_blocks ? n_blocks - 1 : r); };
 
-    constexpr bool kFold = !DROPOUT;
     constexpr float kFoldUnit = 256.f;  // the constant the split terms multiply (keeps f16 terms in range)
     const float neg_inv_c = -1.f / c;
-    f32x16 sc_s, sc_dp;  // S and dP of this member's next block (S - lse / c and dP - delta when folded)
+    f32x16 sc_s, sc_dp;  // S - lse / c and dP - delta of this member's next block
     u32x4 ring[kRing];
     // fragment n of a matrix phase that adds blocks ra and rb and scores block rs
     auto frag = [&](int ra, int rb, int rs, int n) {
@@ -1270,29 +1279,26 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
     auto matrix_phase = [&](auto with_acc, int ra, int rb, int rs) {
         constexpr int first = decltype(with_acc)::value ? 0 : 2 * kAccSteps;
         f32x16 s = zero16(), dp = zero16();
-        // Without dropout one more MFMA each puts -lse / c and -delta under S and dP (a row's value split
-        // into three 16-bit terms against a column of constants), so that the vector phase needs neither
-        // value: P = exp2(c S'), dS = P dP'. Each lane asks for its row's two values at the start.
-        constexpr int kReadStep = first;
+        // One more MFMA each puts -lse / c and -delta under S and dP (a row's value split into three 16-bit
+        // terms against a column of constants), so that the vector phase needs neither value: P = exp2(c S'),
+        // dS = P dP'. Each lane asks for its row's two values at the start of the phase.
         float row_lse = 0.f, row_delta = 0.f;
 #pragma unroll
         for (int n = first; n < kSteps; ++n) {
             const int slot = (n - first) % kRing;
-            if constexpr (kFold) {
-                if (n == kReadStep) {
-                    const float* sLse = reinterpret_cast<const float*>(slot_of(rs) + 2 * kHalfBytes);
-                    row_lse = sLse[l32];
-                    row_delta = sLse[64 + l32];
-                }
-                if (n == 2 * kAccSteps) {
-                    const u32x4 zero4 = {0, 0, 0, 0};
-                    const u32x4 al = split3<T>(row_lse * neg_inv_c * (1.f / kFoldUnit));
-                    const u32x4 ad = split3<T>(row_delta * (-1.f / kFoldUnit));
-                    const uint32_t u2 = Mma<T>::pack2(kFoldUnit, kFoldUnit), u1 = Mma<T>::pack2(kFoldUnit, 0.f);
-                    const u32x4 units = h == 0 ? u32x4{u2, u1, 0, 0} : zero4;
-                    s = Mma<T>::run(h == 0 ? al : zero4, units, s);
-                    dp = Mma<T>::run(h == 0 ? ad : zero4, units, dp);
-                }
+            if (n == first) {
+                const float* sLse = reinterpret_cast<const float*>(slot_of(rs) + 2 * kHalfBytes);
+                row_lse = sLse[l32];
+                row_delta = sLse[64 + l32];
+            }
+            if (n == 2 * kAccSteps) {
+                const u32x4 zero4 = {0, 0, 0, 0};
+                const u32x4 al = split3<T>(row_lse * neg_inv_c * (1.f / kFoldUnit));
+                const u32x4 ad = split3<T>(row_delta * (-1.f / kFoldUnit));
+                const uint32_t u2 = Mma<T>::pack2(kFoldUnit, kFoldUnit), u1 = Mma<T>::pack2(kFoldUnit, 0.f);
+                const u32x4 units = h == 0 ? u32x4{u2, u1, 0, 0} : zero4;
+                s = Mma<T>::run(h == 0 ? al : zero4, units, s);
+                dp = Mma<T>::run(h == 0 ? ad : zero4, units, dp);
             }
             if (n < 2 * kAccSteps) {
                 const int m = n % kAccSteps;
@@ -1316,66 +1322,36 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
 
     // vector phase for block r (this member's): P and dS from sc_s, sc_dp
     constexpr bool kLoadsFirst = CAUSAL;
+    // P = exp2(c S') and dS = P dP' of the block whose first row is rb, eight rows at a time, packed as soon as
+    // they are done; only the block on the diagonal pays for the causal comparison
+    auto softmax_backward = [&](auto on_diagonal, int rb) {
+        const f32x16 s = sc_s, dp = sc_dp;
+#pragma unroll
+        for (int gg = 0; gg < 2; ++gg) {
+            float pr[8], ds[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int i = 8 * gg + j;
+                float pv = fast_exp2(s[i] * c);
+                if constexpr (decltype(on_diagonal)::value) pv = key <= rb + c_row(i, h) ? pv : 0.f;
+                pr[j] = pv;
+                ds[j] = pv * dp[i];
+            }
+            cur_p[gg] = pack8<T>(pr);
+            cur_s[gg] = pack8<T>(ds);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
     auto vector_phase = [&](int r, int ph) {
+        // a load instruction holds the wave until the memory pipeline takes it: with the uneven block counts
+        // of a causal launch it costs least at the start of the phase (measured: 3.6 % fewer cycles than at
+        // the end, where the even non-causal launch does 2 % better)
+        if constexpr (kLoadsFirst) issue_block();
         if (block_on(r)) {
-            const char* slot = slot_of(r);
-            const float* sLse = reinterpret_cast<const float*>(slot + 2 * kHalfBytes);
-            const float* sDelta = sLse + 64;
             const int rb = row_first + r * kBR;
-            const bool diag = CAUSAL && r == kb;
-            const f32x16 s = sc_s, dp = sc_dp;
-            f32x4 lse4[4];
-            if constexpr (!kFold) {
-#pragma unroll
-                for (int g = 0; g < 4; ++g) lse4[g] = *reinterpret_cast<const f32x4*>(sLse + 8 * g + 4 * h);
-            }
-            // a load instruction holds the wave until the memory pipeline takes it: with the uneven block
-            // counts of a causal launch it costs least here, while the lse values are on their way (measured:
-            // 3.6 % fewer cycles than at the end of the phase, where the even non-causal launch does 2 % better)
-            if constexpr (kLoadsFirst) issue_block(ph + 4);
-            Philox4 mine;  // the block of rows rb + 8 (lane % 4) + 4 h .. +3: this lane's share of the quad's four
-            if constexpr (DROPOUT) mine = dropout_block(p, bh, (rb + 8 * (lane & 3) + 4 * h) >> 2, key >> 2);
-#pragma unroll
-            for (int gg = 0; gg < 2; ++gg) {  // eight rows at a time, packed as soon as they are done
-                float pr[8], ds[8];
-                f32x4 dlt4[2];
-#pragma unroll
-                for (int g2 = 0; g2 < 2; ++g2) {
-                    if constexpr (!kFold) dlt4[g2] = *reinterpret_cast<const f32x4*>(sDelta + 8 * (2 * gg + g2) + 4 * h);
-                }
-#pragma unroll
-                for (int g2 = 0; g2 < 2; ++g2) {
-                    const int g = 2 * gg + g2;
-                    const f32x4 l4 = lse4[g];
-                    const f32x4 d4 = dlt4[g2];
-                    uint32_t dw[4];
-                    if constexpr (DROPOUT) {
-                        const Philox4 rr = quad_bcast_from(g, mine);  // lane g of the quad generated rows rb + 8 g + 4 h .. +3
-#pragma unroll
-                        for (int bb = 0; bb < 4; ++bb) dw[bb] = (rr.w[bb] >> (8 * (key & 3))) & 0xffu;
-                    }
-#pragma unroll
-                    for (int bb = 0; bb < 4; ++bb) {
-                        const int i = 4 * g + bb;
-                        float pv = kFold ? fast_exp2(s[i] * c) : fast_exp2(fmaf(s[i], c, -l4[bb]));
-                        if (diag) pv = key <= rb + c_row(i, h) ? pv : 0.f;
-                        float dpv = dp[i];
-                        if constexpr (DROPOUT) {
-                            const bool keep = static_cast<int>(dw[bb]) >= p.thr8;
-                            dpv = keep ? dpv * p.zscale : 0.f;
-                            pr[4 * g2 + bb] = keep ? pv * p.zscale : 0.f;
-                        } else {
-                            pr[4 * g2 + bb] = pv;
-                        }
-                        ds[4 * g2 + bb] = kFold ? pv * dpv : pv * (dpv - d4[bb]);
-                    }
-                }
-                cur_p[gg] = pack8<T>(pr);
-                cur_s[gg] = pack8<T>(ds);
-                __builtin_amdgcn_sched_barrier(0);
-            }
+            if (CAUSAL && r == kb) softmax_backward(Yes{}, rb);
+            else softmax_backward(No{}, rb);
         } else {
-            if constexpr (kLoadsFirst) issue_block(ph + 4);
 #pragma unroll
             for (int g = 0; g < 2; ++g) cur_p[g] = cur_s[g] = u32x4{0, 0, 0, 0};
         }
@@ -1388,7 +1364,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
             *reinterpret_cast<u32x4*>(my_xch + g * 1024) = cur_p[g];
             *reinterpret_cast<u32x4*>(my_xch + (2 + g) * 1024) = cur_s[g];
         }
-        if constexpr (!kLoadsFirst) issue_block(ph + 4);
+        if constexpr (!kLoadsFirst) issue_block();
         asm volatile("" ::: "memory");  // the reads below are issued after the writes above
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
@@ -1412,14 +1388,14 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
         __builtin_amdgcn_s_setprio(2);
         matrix_phase(Yes{}, clamp_block(r - 1), clamp_block(r), r + 2);
         __builtin_amdgcn_s_setprio(0);
-        issue_block(ph + 4);
+        issue_block();
         wait_blocks(ph);
         __builtin_amdgcn_sched_barrier(0);
         lds_barrier();
         __builtin_amdgcn_sched_barrier(0);
     };
     auto idle_phase = [&](int ph) {
-        issue_block(ph + 4);
+        issue_block();
         wait_blocks(ph);
         lds_barrier();
     };
@@ -1529,7 +1505,7 @@ int launch_dkdv_dropout(const KParams& p, hipStream_t stream) {
         const dim3 grid(p.B * p.H * (p.S / kBM)), block(512);
         if constexpr (MASK == kNoMask) {
             if (p.thr8 <= 0) {
-                hipLaunchKernelGGL((mfma_dkdv_phased_kernel<T, D, CAUSAL, false>), grid, block, 0, stream, p);
+                hipLaunchKernelGGL((mfma_dkdv_phased_kernel<T, D, CAUSAL>), grid, block, 0, stream, p);
                 return static_cast<int>(hipGetLastError());
             }
         }
