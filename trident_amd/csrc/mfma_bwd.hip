@@ -196,13 +196,17 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
             for (int i = 0; i < 2 * DB; ++i)
                 tf[i] = Tile::tr_frag(sK, tr_off0 ^ ((i % DB) << 6), tr_off1 ^ ((i % DB) << 6), 2 * kb + i / DB);
             __builtin_amdgcn_sched_barrier(0);
+            if (diag && t0 + 32 * kb + 31 > wrow0) {  // a block that crosses the diagonal: scores above it drop out
+                asm volatile("");                     // (a real branch: the other blocks skip the comparisons)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) st[i] = t0 + 32 * kb + c_row(i, h) <= qrow ? st[i] : -INFINITY;
+            }
             float ds[16];
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 float pr;
                 if constexpr (MASK != kNoMask) pr = fast_exp2(fmaf(mk[i], kLog2e, st[i] * c) - lse);
                 else pr = fast_exp2(fmaf(st[i], c, -lse));
-                if (diag) pr = t0 + 32 * kb + c_row(i, h) <= qrow ? pr : 0.f;
                 ds[i] = pr;
             }
             if constexpr (DROPOUT) {
@@ -414,16 +418,15 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
     for (int t = 0; t < my_tiles; ++t) {
         const bool issued = t + dist < n_tiles;
         if (issued) issue_tile(t + dist);
-        // ---- vector phase: P and dS of the tile
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
+        // ---- vector phase: P and dS of the tile (only 32-key blocks that cross the diagonal pay for the
+        // causal comparison)
+        auto softmax_backward = [&](auto on_diagonal, int kb) {
             const int key0 = t * kBN + 32 * kb;
-            const bool diag = CAUSAL && key0 + 31 > wrow0;
             float ds[16];
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 float pr = fast_exp2(fmaf(st[kb][i], c, -lse));
-                if (diag) pr = key0 + c_row(i, h) <= qrow ? pr : 0.f;
+                if constexpr (decltype(on_diagonal)::value) pr = key0 + c_row(i, h) <= qrow ? pr : 0.f;
                 ds[i] = pr;
             }
             f32x16 dpv = dpt[kb];
@@ -443,6 +446,11 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
             for (int i = 0; i < 16; ++i) ds[i] *= dpv[i] - dlt;
             bop[2 * kb + 0] = pack8<T>(&ds[0]);
             bop[2 * kb + 1] = pack8<T>(&ds[8]);
+        };
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            if (CAUSAL && t * kBN + 32 * kb + 31 > wrow0) softmax_backward(Yes{}, kb);
+            else softmax_backward(No{}, kb);
         }
         // the first fragments of the matrix phase (K^T of this tile, visible since the previous barrier)
 #pragma unroll
@@ -654,6 +662,11 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
 #pragma unroll
             for (int kk = 0; kk < KK; ++kk) dp = Mma<T>::run(fr[kk], vf[kk], dp);
             __builtin_amdgcn_sched_barrier(0);
+            if (diag && rb < wkey0 + 31) {  // a block that crosses the diagonal: scores above it drop out
+                asm volatile("");           // (a real branch: the other blocks skip the comparisons)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) s[i] = key <= rb + c_row(i, h) ? s[i] : -INFINITY;
+            }
             u32x4 pb[2], sb[2];
             {
                 float pr[16], ds[16];
@@ -679,7 +692,6 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
                         float pv;
                         if constexpr (MASK != kNoMask) pv = fast_exp2(fmaf(mk[i], kLog2e, s[i] * c) - l4[bb]);
                         else pv = fast_exp2(fmaf(s[i], c, -l4[bb]));
-                        if (diag) pv = key <= rb + c_row(i, h) ? pv : 0.f;
                         float dpv = dp[i];
                         if constexpr (DROPOUT) {
                             const bool keep = static_cast<int>(dw[bb]) >= p.thr8;
@@ -953,8 +965,13 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
             const char* sQ = smem + (lt % kStages) * kStageBytes;
             const char* sG = sQ + Tile::kBytes;
             const float* sDelta = reinterpret_cast<const float*>(sG + Tile::kBytes) + kBN;
-            const bool diag = CAUSAL && rb < wkey0 + 31;
-            const f32x16 s = sc_s, dp = sc_dp;
+            f32x16 s = sc_s;
+            const f32x16 dp = sc_dp;
+            if (CAUSAL && rb < wkey0 + 31) {  // a block that crosses the diagonal: scores above it drop out
+                asm volatile("");             // (a real branch: the other blocks skip the comparisons)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) s[i] = key <= rb + c_row(i, h) ? s[i] : -INFINITY;
+            }
             float mk[MASK != kNoMask ? 16 : 1];
             if constexpr (MASK != kNoMask) {
                 const int64_t mbase = b * p.ms[0] + hd * p.ms[1] + key;
@@ -994,7 +1011,6 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
                         float pv;
                         if constexpr (MASK != kNoMask) pv = fast_exp2(fmaf(mk[i], kLog2e, s[i] * c) - l4[bb]);
                         else pv = fast_exp2(fmaf(s[i], c, -l4[bb]));
-                        if (diag) pv = key <= rb + c_row(i, h) ? pv : 0.f;
                         float dpv = dp[i];
                         if constexpr (DROPOUT) {
                             const bool keep = static_cast<int>(dw[bb]) >= p.thr8;
