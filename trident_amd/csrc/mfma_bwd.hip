@@ -271,7 +271,16 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
     constexpr int kSteps = kDqSteps + 4 * KK;  // + S^T and dP^T of the next tile
     constexpr int kRing = 6;
     static_assert(kRing <= kDqSteps, "the vector phase requests dQ fragments only");
-    __shared__ __attribute__((aligned(1024))) char smem[kStages * kStageBytes];
+    // The workgroup's Q and dO rows reach the registers through LDS as well: lanes own rows, so direct loads
+    // touch 32 cache lines per instruction, while LDS-direct loads fetch whole rows. Each wave stages its
+    // own 32 rows behind ring stage 0, which takes tile 0 meanwhile; tiles 1 and 2 follow once every wave
+    // has its rows. The O rows (for delta) do come by direct loads, issued first: LDS has no room for a
+    // third operand at once, and staging O after Q in a second round trip measured the same. What remains
+    // of a workgroup's start is the latency of its first loads (about 6 000 cycles for a single plain load).
+    constexpr int kWaveRowBytes = 32 * Tile::kRowBytes;  // a wave's rows of one operand
+    constexpr int kRowLoads = kWaveRowBytes / 1024;      // LDS-direct loads per wave and operand
+    __shared__ __attribute__((aligned(1024))) char smem[kStageBytes + 2 * NW * kWaveRowBytes];
+    static_assert(kStageBytes + 2 * NW * kWaveRowBytes >= kStages * kStageBytes, "the ring lies inside");
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -283,28 +292,29 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
     const int wrow0 = q0 + 32 * wave;
     const int qrow = wrow0 + l32;
 
-    const char* qrowp = static_cast<const char*>(p.q) + (b * p.qs[0] + hd * p.qs[1] + static_cast<int64_t>(qrow) * p.qs[2]) * 2;
-    const char* gorowp = static_cast<const char*>(p.d_o) + (b * p.dos[0] + hd * p.dos[1] + static_cast<int64_t>(qrow) * p.dos[2]) * 2;
+    const char* qrows = static_cast<const char*>(p.q) + (b * p.qs[0] + hd * p.qs[1] + static_cast<int64_t>(wrow0) * p.qs[2]) * 2;
+    const char* gorows = static_cast<const char*>(p.d_o) + (b * p.dos[0] + hd * p.dos[1] + static_cast<int64_t>(wrow0) * p.dos[2]) * 2;
     const char* kbase = static_cast<const char*>(p.k) + (b * p.ks[0] + hd * p.ks[1]) * 2;
     const char* vbase = static_cast<const char*>(p.v) + (b * p.vs[0] + hd * p.vs[1]) * 2;
     const int64_t krow_bytes = p.ks[2] * 2, vrow_bytes = p.vs[2] * 2;
 
-    u32x4 qf[KK], gf[KK];
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-        qf[kk] = *reinterpret_cast<const u32x4*>(qrowp + (2 * kk + h) * 16);
-        gf[kk] = *reinterpret_cast<const u32x4*>(gorowp + (2 * kk + h) * 16);
-    }
+    float lse = p.lse[static_cast<int64_t>(bh) * p.S + qrow];
+    float dlt = 0.f;
+    if constexpr (!DELTA) dlt = p.delta[static_cast<int64_t>(bh) * p.S + qrow];
     u32x4 of[DELTA ? KK : 1];
     if constexpr (DELTA) {
         const char* orowp = static_cast<const char*>(p.o) + (b * p.os[0] + hd * p.os[1] + static_cast<int64_t>(qrow) * p.os[2]) * 2;
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) of[kk] = *reinterpret_cast<const u32x4*>(orowp + (2 * kk + h) * 16);
     }
-    float lse = p.lse[static_cast<int64_t>(bh) * p.S + qrow];
-    if (lse == -INFINITY) lse = INFINITY;  // fully masked row: every probability is 0
-    float dlt = 0.f;
-    if constexpr (!DELTA) dlt = p.delta[static_cast<int64_t>(bh) * p.S + qrow];
+    char* q_stage = smem + kStageBytes + wave * kWaveRowBytes;
+    char* g_stage = q_stage + NW * kWaveRowBytes;
+#pragma unroll
+    for (int blk = 0; blk < kRowLoads; ++blk)
+        lds_direct_load16(qrows, static_cast<uint32_t>(Tile::src_off(blk, lane, p.qs[2] * 2)), q_stage + blk * 1024);
+#pragma unroll
+    for (int blk = 0; blk < kRowLoads; ++blk)
+        lds_direct_load16(gorows, static_cast<uint32_t>(Tile::src_off(blk, lane, p.dos[2] * 2)), g_stage + blk * 1024);
     const float c = p.scale_log2;
 
     f32x16 acc[DB];
@@ -332,32 +342,32 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
     const int dist = 2 + group;
     const int n_first = min(dist, n_tiles);
     issue_tile(0);
-    if (n_first > 1) issue_tile(1);
-    if (n_first > 2) issue_tile(2);
-    // (the row fragments were requested before the tiles, so both latencies overlap)
+
+    const int row_off0 = Tile::off(l32, h);
+    TRI_WAIT_VMCNT(kBlocksPerWave);  // this wave's Q and dO rows have landed (tile 0 may be on its way)
+    asm volatile("" ::: "memory");
+    u32x4 qf[KK], gf[KK];
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
-        settle(qf[kk]);
-        settle(gf[kk]);
+        qf[kk] = lds_read16(q_stage, row_off0 ^ (kk << 5));
+        gf[kk] = lds_read16(g_stage, row_off0 ^ (kk << 5));
     }
-    settle(lse);
     if constexpr (DELTA) {
         // this lane holds half of its row (the other half is in lane ^ 32)
         float part = 0.f;
 #pragma unroll
-        for (int kk = 0; kk < KK; ++kk)
+        for (int kk = 0; kk < KK; ++kk) {
+            settle(of[kk]);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 part = fmaf(Mma<T>::lo(of[kk][i]), Mma<T>::lo(gf[kk][i]), part);
                 part = fmaf(Mma<T>::hi(of[kk][i]), Mma<T>::hi(gf[kk][i]), part);
             }
+        }
         dlt = sum_xor32(part);
         if (h == 0) p.delta[static_cast<int64_t>(bh) * p.S + qrow] = dlt;
-    } else {
-        settle(dlt);
     }
 
-    const int row_off0 = Tile::off(l32, h);
     const int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
 
     // fragment n of the matrix phase of tile t: n < kDqSteps: K^T of tile t (column block n % DB, K-step
@@ -397,11 +407,15 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
         else TRI_WAIT_VMCNT(0);
     };
 
-    // tile 0 has landed and is visible to all waves
-    if (n_first == 3) TRI_WAIT_VMCNT(2 * kBlocksPerWave);
-    else if (n_first == 2) TRI_WAIT_VMCNT(kBlocksPerWave);
-    else TRI_WAIT_VMCNT(0);
+    // tile 0 has landed and is visible to all waves, and every wave has its rows in registers: the staging
+    // area returns to the ring
+    TRI_WAIT_VMCNT(0);
+    settle(lse);
+    if constexpr (!DELTA) settle(dlt);
+    if (lse == -INFINITY) lse = INFINITY;  // fully masked row: every probability is 0
     lds_barrier();
+    if (n_first > 1) issue_tile(1);
+    if (n_first > 2) issue_tile(2);
     if (group == 1) {
         // group 1 starts one phase late; group 0 reads tile 1 in its first matrix phase
         if (n_first == 3) TRI_WAIT_VMCNT(kBlocksPerWave);
@@ -1336,8 +1350,6 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
     using Yes = std::integral_constant<bool, true>;
     using No = std::integral_constant<bool, false>;
 
-    // vector phase for block r (this member's): P and dS from sc_s, sc_dp
-    constexpr bool kLoadsFirst = CAUSAL;
     // P = exp2(c S') and dS = P dP' of the block whose first row is rb, eight rows at a time, packed as soon as
     // they are done; only the block on the diagonal pays for the causal comparison
     auto softmax_backward = [&](auto on_diagonal, int rb) {
@@ -1358,11 +1370,8 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    auto vector_phase = [&](int r, int ph) {
-        // a load instruction holds the wave until the memory pipeline takes it: with the uneven block counts
-        // of a causal launch it costs least at the start of the phase (measured: 3.6 % fewer cycles than at
-        // the end, where the even non-causal launch does 2 % better)
-        if constexpr (kLoadsFirst) issue_block();
+    // vector phase for block r (this member's): P and dS from sc_s, sc_dp
+    auto vector_phase = [&](int r) {
         if (block_on(r)) {
             const int rb = row_first + r * kBR;
             if (CAUSAL && r == kb) softmax_backward(Yes{}, rb);
@@ -1380,7 +1389,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
             *reinterpret_cast<u32x4*>(my_xch + g * 1024) = cur_p[g];
             *reinterpret_cast<u32x4*>(my_xch + (2 + g) * 1024) = cur_s[g];
         }
-        if constexpr (!kLoadsFirst) issue_block();
+        issue_block();
         asm volatile("" ::: "memory");  // the reads below are issued after the writes above
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
@@ -1429,7 +1438,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
 #pragma unroll 1
         for (int t = 0; t <= n_iter; ++t) {   // the last round only adds member 1's last block
             const int r = 2 * t;
-            vector_phase(r, 2 * t);
+            vector_phase(r);
             close_vector_phase(2 * t, r);
             run_matrix_phase(2 * t + 1, r);
         }
@@ -1438,7 +1447,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
 #pragma unroll 1
         for (int t = 0; t < n_iter; ++t) {
             const int r = 2 * t + 1;
-            vector_phase(r, 2 * t + 1);
+            vector_phase(r);
             close_vector_phase(2 * t + 1, r);
             run_matrix_phase(2 * t + 2, r);
         }
