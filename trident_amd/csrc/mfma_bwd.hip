@@ -274,9 +274,10 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
     // The workgroup's Q and dO rows reach the registers through LDS as well: lanes own rows, so direct loads
     // touch 32 cache lines per instruction, while LDS-direct loads fetch whole rows. Each wave stages its
     // own 32 rows behind ring stage 0, which takes tile 0 meanwhile; tiles 1 and 2 follow once every wave
-    // has its rows. The O rows (for delta) do come by direct loads, issued first: LDS has no room for a
-    // third operand at once, and staging O after Q in a second round trip measured the same. What remains
-    // of a workgroup's start is the latency of its first loads (about 6 000 cycles for a single plain load).
+    // has its rows. The O rows (for delta) take the place of the Q rows in a second round (LDS has no room
+    // for a third operand at once; fetching them by direct loads during the first round measured 1 %
+    // slower). What remains of a workgroup's start is the latency of its first loads (about 6 000 cycles
+    // for a single plain load).
     constexpr int kWaveRowBytes = 32 * Tile::kRowBytes;  // a wave's rows of one operand
     constexpr int kRowLoads = kWaveRowBytes / 1024;      // LDS-direct loads per wave and operand
     __shared__ __attribute__((aligned(1024))) char smem[kStageBytes + 2 * NW * kWaveRowBytes];
@@ -301,12 +302,6 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
     float lse = p.lse[static_cast<int64_t>(bh) * p.S + qrow];
     float dlt = 0.f;
     if constexpr (!DELTA) dlt = p.delta[static_cast<int64_t>(bh) * p.S + qrow];
-    u32x4 of[DELTA ? KK : 1];
-    if constexpr (DELTA) {
-        const char* orowp = static_cast<const char*>(p.o) + (b * p.os[0] + hd * p.os[1] + static_cast<int64_t>(qrow) * p.os[2]) * 2;
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) of[kk] = *reinterpret_cast<const u32x4*>(orowp + (2 * kk + h) * 16);
-    }
     char* q_stage = smem + kStageBytes + wave * kWaveRowBytes;
     char* g_stage = q_stage + NW * kWaveRowBytes;
 #pragma unroll
@@ -353,15 +348,23 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
         gf[kk] = lds_read16(g_stage, row_off0 ^ (kk << 5));
     }
     if constexpr (DELTA) {
-        // this lane holds half of its row (the other half is in lane ^ 32)
+        // the O rows follow into the place of the Q rows; this lane holds half of its row (the other half is
+        // in lane ^ 32)
+        const char* orows = static_cast<const char*>(p.o) + (b * p.os[0] + hd * p.os[1] + static_cast<int64_t>(wrow0) * p.os[2]) * 2;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the Q rows are in registers
+#pragma unroll
+        for (int blk = 0; blk < kRowLoads; ++blk)
+            lds_direct_load16(orows, static_cast<uint32_t>(Tile::src_off(blk, lane, p.os[2] * 2)), q_stage + blk * 1024);
+        TRI_WAIT_VMCNT(0);
+        asm volatile("" ::: "memory");
         float part = 0.f;
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) {
-            settle(of[kk]);
+            const u32x4 of = lds_read16(q_stage, row_off0 ^ (kk << 5));
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                part = fmaf(Mma<T>::lo(of[kk][i]), Mma<T>::lo(gf[kk][i]), part);
-                part = fmaf(Mma<T>::hi(of[kk][i]), Mma<T>::hi(gf[kk][i]), part);
+                part = fmaf(Mma<T>::lo(of[i]), Mma<T>::lo(gf[kk][i]), part);
+                part = fmaf(Mma<T>::hi(of[i]), Mma<T>::hi(gf[kk][i]), part);
             }
         }
         dlt = sum_xor32(part);
