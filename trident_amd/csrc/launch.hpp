@@ -21,5 +21,8 @@ int launch_mfma_dq(int dtype, const KParams& p, hipStream_t stream, bool with_de
 bool mfma_dq_fuses_delta(const KParams& p);
 int launch_mfma_dkdv(int dtype, const KParams& p, hipStream_t stream);
 int launch_delta(int dtype, const KParams& p, hipStream_t stream);
+// Number of workgroups for a kernel whose workgroups are persistent (one per CU, each walking several of
+// the `items`): min(items, CUs of the current device).
+int persistent_grid(int items);
 
 }  // namespace tri

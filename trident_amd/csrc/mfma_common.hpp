@@ -250,6 +250,27 @@ __device__ __forceinline__ void map_block_shared_mask(int bid, int batches, int 
     *tile = unit % num_tiles;
 }
 
+// Persistent workgroups: a launch of `grid` workgroups (one per CU) walks the head x tile items in rounds;
+// workgroup `bid` takes one item per round and the function says whether round `round` still has one for it.
+// The items of an XCD are those map_block gives its workgroups, in the same order (heaviest tiles first
+// under a causal mask, head after head otherwise); odd rounds hand them out in reverse, so that a
+// workgroup with a heavy item in one round gets a light one in the next and all finish together.
+__device__ __forceinline__ bool map_item(int bid, int grid, int round, int num_heads, int num_tiles, int order,
+                                         int* bh, int* tile) {
+    const int items = num_heads * num_tiles;
+    if ((num_heads & 7) == 0 && (grid & 7) == 0) {
+        const int xcd = bid & 7, slot = bid >> 3, per_round = grid >> 3;
+        const int j = round * per_round + ((round & 1) ? per_round - 1 - slot : slot);
+        if (j >= (items >> 3)) return false;
+        map_block(j * 8 + xcd, num_heads, num_tiles, order, bh, tile);
+        return true;
+    }
+    const int j = round * grid + bid;
+    if (j >= items) return false;
+    map_block(j, num_heads, num_tiles, order, bh, tile);
+    return true;
+}
+
 template <int MASK>
 __device__ __forceinline__ void map_block_for(const KParams& p, int bid, int num_tiles, int order, int* bh, int* tile) {
     if (MASK != 0 && p.ms[1] == 0 && p.H > 1) map_block_shared_mask(bid, p.B, p.H, num_tiles, bh, tile);

@@ -52,35 +52,50 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     constexpr bool kMaskViaLds = MASK == kMaskF32 && D == 64;
     using MaskTile = SwzTile<128>;
     constexpr int kMaskBytes = 32 * MaskTile::kRowBytes;
-    __shared__ __attribute__((aligned(1024))) char smem[kStages * kStageBytes + (kMaskViaLds ? NW * kMaskBytes : 0)];
+    // Without an additive mask the 8-wave kernel is persistent: one workgroup per CU walks several (head, row
+    // tile) items, and requests the Q rows and the first tiles of its next item before it stores the current
+    // one, so that a new item's memory latency (6 000-9 000 cycles from a workgroup's entry to its first rows)
+    // passes behind the epilogue. The epilogue's transposition patches then must not lie in ring stages 0-2.
+    constexpr bool kPersistent = NW == 8 && MASK == kNoMask;
+    using Store = RowBlockStore<T, 2>;                       // the epilogue stores 64 columns at a time
+    constexpr int kPatchOff = kPersistent ? 3 * kStageBytes : 0;
+    constexpr int kRingBytes = kStages * kStageBytes;
+    constexpr int kPatchEnd = kPatchOff + NW * Store::kPatchBytes;
+    constexpr int kSmemBytes = (kPatchEnd > kRingBytes ? kPatchEnd : kRingBytes) + (kMaskViaLds ? NW * kMaskBytes : 0);
+    __shared__ __attribute__((aligned(1024))) char smem[kSmemBytes];
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+    // the current item (head bh, row tile qt) and what follows from it
+    constexpr int kOrder = CAUSAL ? kHeavyLast : kUniformTiles;
+    int round = 0;
     int bh, qt;
-    map_block_for<MASK>(p, blockIdx.x, p.S / kBM, CAUSAL ? kHeavyLast : kUniformTiles, &bh, &qt);
-    const int b = bh / p.H, hd = bh % p.H;
-    const int q0 = qt * kBM;
-    const int wrow0 = q0 + 32 * wave;  // first query row of this wave
-    const int qrow = wrow0 + l32;
-
-    const char* qbase = static_cast<const char*>(p.q) + (b * p.qs[0] + hd * p.qs[1]) * 2;
-    const char* kbase = static_cast<const char*>(p.k) + (b * p.ks[0] + hd * p.ks[1]) * 2;
-    const char* vbase = static_cast<const char*>(p.v) + (b * p.vs[0] + hd * p.vs[1]) * 2;
+    if constexpr (kPersistent) map_item(blockIdx.x, gridDim.x, 0, p.B * p.H, p.S / kBM, kOrder, &bh, &qt);
+    else map_block_for<MASK>(p, blockIdx.x, p.S / kBM, kOrder, &bh, &qt);
+    int b, hd, wrow0, qrow, n_tiles, my_tiles;
+    const char *kbase, *vbase;
     const int64_t krow_bytes = p.ks[2] * 2, vrow_bytes = p.vs[2] * 2;
-
     u32x4 qf[KK];
+    auto set_item = [&]() {  // (also requests the item's Q rows)
+        b = bh / p.H;
+        hd = bh % p.H;
+        const int q0 = qt * kBM;
+        wrow0 = q0 + 32 * wave;  // first query row of this wave
+        qrow = wrow0 + l32;
+        const char* qbase = static_cast<const char*>(p.q) + (b * p.qs[0] + hd * p.qs[1]) * 2;
+        kbase = static_cast<const char*>(p.k) + (b * p.ks[0] + hd * p.ks[1]) * 2;
+        vbase = static_cast<const char*>(p.v) + (b * p.vs[0] + hd * p.vs[1]) * 2;
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk)
-        qf[kk] = *reinterpret_cast<const u32x4*>(qbase + qrow * p.qs[2] * 2 + (2 * kk + h) * 16);
+        for (int kk = 0; kk < KK; ++kk)
+            qf[kk] = *reinterpret_cast<const u32x4*>(qbase + qrow * p.qs[2] * 2 + (2 * kk + h) * 16);
+        n_tiles = CAUSAL ? (q0 + kBM) / kBN : p.S / kBN;       // tiles the workgroup streams
+        my_tiles = CAUSAL ? (wrow0 + 31) / kBN + 1 : n_tiles;  // tiles this wave has visible keys in
+    };
+    set_item();
 
     f32x16 oacc[DB];
-#pragma unroll
-    for (int db = 0; db < DB; ++db) oacc[db] = zero16();
-    float m = -INFINITY, l = 0.f;  // reference exponent (log2 domain, scaled) and this lane's partial sum
-
-    const int n_tiles = CAUSAL ? (q0 + kBM) / kBN : p.S / kBN;            // tiles the workgroup streams
-    const int my_tiles = CAUSAL ? (wrow0 + 31) / kBN + 1 : n_tiles;       // tiles this wave has visible keys in
+    float m, l;  // reference exponent (log2 domain, scaled) and this lane's partial sum
     const float c = p.scale_log2;
 
     char* mask_lds = smem + kStages * kStageBytes + wave * kMaskBytes;
@@ -141,13 +156,14 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
         else if (tile) TRI_WAIT_VMCNT(kB);
         else TRI_WAIT_VMCNT(0);
     };
-    const int n_first = min(dist, n_tiles);
-    issue_tile(0);
-    if (n_first > 1) issue_tile(1);
-    if (n_first > 2) issue_tile(2);
-    // (the Q fragments were requested before the tiles, so both latencies overlap)
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) settle(qf[kk]);
+    int n_first;
+    auto request_first_tiles = [&]() {  // (the Q rows were requested before, so both latencies overlap)
+        n_first = min(dist, n_tiles);
+        issue_tile(0);
+        if (n_first > 1) issue_tile(1);
+        if (n_first > 2) issue_tile(2);
+    };
+    request_first_tiles();
 
     int row_off0 = Tile::off(l32, h);
     int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
@@ -266,14 +282,24 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     using Yes = std::integral_constant<bool, true>;
     using No = std::integral_constant<bool, false>;
 
-    // tile 0 has landed and is visible to all waves
-    if (n_first == 3) TRI_WAIT_VMCNT(2 * kBlocksPerWave);
+    for (bool first_item = true;; first_item = false) {  // one pass per item
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) settle(qf[kk]);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) oacc[db] = zero16();
+    lacc = zero16();
+    m = -INFINITY;
+    l = 0.f;
+    // tile 0 has landed and is visible to all waves (a later item's requests are older than the stores of the
+    // item before it: everything is awaited)
+    if (!first_item) TRI_WAIT_VMCNT(0);
+    else if (n_first == 3) TRI_WAIT_VMCNT(2 * kBlocksPerWave);
     else if (n_first == 2) TRI_WAIT_VMCNT(kBlocksPerWave);
     else TRI_WAIT_VMCNT(0);
     lds_barrier();
     if (kPingPong && group == 1) {
         // group 1 starts one phase late; group 0 reads tile 1 in its first matrix phase
-        if (n_first == 3) TRI_WAIT_VMCNT(kBlocksPerWave);
+        if (first_item && n_first == 3) TRI_WAIT_VMCNT(kBlocksPerWave);
         else TRI_WAIT_VMCNT(0);
         lds_barrier();
     }
@@ -436,20 +462,39 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
 
     l = DROPOUT ? sum_xor32(l) : lacc[0];
     const float inv = 1.f / l;
-    // every wave is out of the loop: the ring can serve as the waves' private transposition patches
+    // every wave is out of the loop: the ring is free (for the waves' private transposition patches, and for
+    // the first tiles of the next item)
     lds_barrier();
-    {
-        using Store = RowBlockStore<T, DB>;
-        static_assert(NW * Store::kPatchBytes <= kStages * kStageBytes, "patches must fit into the ring");
-        char* o0 = static_cast<char*>(p.o) + (b * p.os[0] + hd * p.os[1] + static_cast<int64_t>(wrow0) * p.os[2]) * 2;
-        Store::run(oacc, [inv](float x) { return x * inv; }, smem + wave * Store::kPatchBytes, o0, p.os[2] * 2, lane);
+    char* o0 = static_cast<char*>(p.o) + (b * p.os[0] + hd * p.os[1] + static_cast<int64_t>(wrow0) * p.os[2]) * 2;
+    float* lse_out = p.lse + static_cast<int64_t>(bh) * p.S + qrow;
+    bool more = false;
+    if constexpr (kPersistent) {
+        more = map_item(blockIdx.x, gridDim.x, ++round, p.B * p.H, p.S / kBM, kOrder, &bh, &qt);
+        if (more) {
+            set_item();
+            request_first_tiles();
+        }
     }
-    if (h == 0) p.lse[static_cast<int64_t>(bh) * p.S + qrow] = m + fast_log2(l);
+    {
+        static_assert(DB % 2 == 0, "64 columns per store");
+        char* patch = smem + kPatchOff + wave * Store::kPatchBytes;
+#pragma unroll
+        for (int cb = 0; cb < DB / 2; ++cb) {
+            if (cb) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // patch read before it is rewritten
+            const f32x16(&part)[2] = *reinterpret_cast<const f32x16(*)[2]>(&oacc[2 * cb]);
+            Store::run(part, [inv](float x) { return x * inv; }, patch, o0 + cb * 128, p.os[2] * 2, lane);
+        }
+    }
+    if (h == 0) *lse_out = m + fast_log2(l);
+    if (!more) break;
+    }
 }
 
 template <typename T, int D, int NW, bool CAUSAL, int MASK>
 int launch_fwd_dropout(const KParams& p, hipStream_t stream) {
-    const dim3 grid(p.B * p.H * (p.S / (32 * NW))), block(64 * NW);
+    const int items = p.B * p.H * (p.S / (32 * NW));
+    // (the kernel's kPersistent: one workgroup per CU walks the items)
+    const dim3 grid(NW == 8 && MASK == kNoMask ? persistent_grid(items) : items), block(64 * NW);
     if (p.thr8 > 0) hipLaunchKernelGGL((mfma_fwd_kernel<T, D, NW, CAUSAL, MASK, true>), grid, block, 0, stream, p);
     else hipLaunchKernelGGL((mfma_fwd_kernel<T, D, NW, CAUSAL, MASK, false>), grid, block, 0, stream, p);
     return static_cast<int>(hipGetLastError());

@@ -87,6 +87,18 @@ bool mfma_dq_fuses_delta(const KParams& p) {
     return aligned16(p.o) && strides8(p.os);
 }
 
+int persistent_grid(int items) {
+    static int cus[64] = {};  // per device ordinal; 0 = not asked yet
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return items;
+    if (cus[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return items;
+        cus[dev] = n;
+    }
+    return items < cus[dev] ? items : cus[dev];
+}
+
 int launch_delta(int dtype, const KParams& p, hipStream_t stream) {
     const bool vec = (dtype == TRI_ATTN_F16 || dtype == TRI_ATTN_BF16) && (p.D == 64 || p.D == 128) &&
                      aligned16(p.o) && aligned16(p.d_o) && strides8(p.os) && strides8(p.dos) &&
