@@ -253,17 +253,17 @@ def test_dropout_extremes_and_determinism(device):
 
 
 # ------------------------------------------------------------------ lengths the operator API rejects
-def _abi_case(device, dtype, S, D, variant, seed):
+def _abi_case(device, dtype, S, D, variant, seed, batches=1, heads=2):
     """The operator API accepts power-of-two lengths only (reference rule); the C ABI takes any
     length.  This calls the ABI wrappers directly: a multiple of 128 that is not one of 256 runs the
     4-wave matrix-core kernels over several tiles, other lengths run the general kernels."""
     from trident_amd.operation import Attention
-    q, k, v, d_o = _gen((1, 2, S, D), seed, dtype)
+    q, k, v, d_o = _gen((batches, heads, S, D), seed, dtype)
     mask, causal, p = None, False, 0.0
     if variant == "causal":
         causal = True
     elif variant == "mask":
-        mask = torch.randn(1, 2, S, S, generator=torch.Generator().manual_seed(seed + 1))
+        mask = torch.randn(batches, heads, S, S, generator=torch.Generator().manual_seed(seed + 1))
     elif variant == "mask16":
         mask = torch.randn(1, 1, S, S, generator=torch.Generator().manual_seed(seed + 1)).to(dtype)
     elif variant == "causal+dropout":
@@ -306,6 +306,15 @@ def test_phased_kernels_over_tile_counts(S, D, variant, device):
     streamed tiles, so the prologue, the steady state and the drain of the load pipeline of the forward
     and dQ kernels, and the waves that stop early under the causal mask, are all exercised."""
     _abi_case(device, torch.bfloat16 if D == 128 else torch.float16, S, D, variant, 500 + S + D)
+
+
+@pytest.mark.parametrize("variant", ["plain", "causal", "causal+dropout"])
+@pytest.mark.parametrize("batches,heads,S,D", [(4, 40, 512, 128), (3, 31, 768, 64), (8, 8, 1280, 128)])
+def test_more_items_than_compute_units(batches, heads, S, D, variant, device):
+    """More (head, row tile) items than the GPU has compute units (320, 279 and 320 against 256): the
+    persistent forward workgroups each walk two items, with the items dealt per XCD when the head count is a
+    multiple of 8 (a partly filled, reversed second round) and in launch order otherwise."""
+    _abi_case(device, torch.bfloat16 if D == 128 else torch.float16, S, D, variant, 700 + S + D, batches, heads)
 
 
 # ------------------------------------------------------------------ the combined backward entry point
