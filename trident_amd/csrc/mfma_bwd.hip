@@ -269,7 +269,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
     static_assert(kRowStep % 16 == 0 && 2 * kPerOperand == kBlocksPerWave, "block assignment");
     constexpr int kDqSteps = 4 * DB;           // MFMAs of dQ^T per tile
     constexpr int kSteps = kDqSteps + 4 * KK;  // + S^T and dP^T of the next tile
-    constexpr int kRing = 6;
+    constexpr int kRing = DROPOUT && D == 128 ? 4 : 6;  // (registers)
     static_assert(kRing <= kDqSteps, "the vector phase requests dQ fragments only");
     // The workgroup's Q and dO rows reach the registers through LDS as well: lanes own rows, so direct loads
     // touch 32 cache lines per instruction, while LDS-direct loads fetch whole rows. Each wave stages its
@@ -1482,11 +1482,11 @@ int launch_dq_waves(const KParams& p, hipStream_t stream) {
     return static_cast<int>(hipGetLastError());
 }
 
-// whether the phased dQ kernel serves this problem (no mask, 256-row workgroups; with dropout at D = 128 it
-// would not fit its registers)
+// whether the phased dQ kernel serves this problem (no mask, 256-row workgroups; with dropout at D = 128 it fits
+// its registers only under the causal mask and with a fragment ring of 4)
 template <int D, int MASK>
 bool dq_is_phased(const KParams& p) {
-    return MASK == kNoMask && p.S % 256 == 0 && (D == 64 || p.thr8 <= 0);
+    return MASK == kNoMask && p.S % 256 == 0 && (D == 64 || p.thr8 <= 0 || p.causal);
 }
 
 template <typename T, int D, bool CAUSAL, int MASK>
@@ -1494,7 +1494,7 @@ int launch_dq_dropout(const KParams& p, hipStream_t stream, bool with_delta) {
     if constexpr (MASK == kNoMask) {
         if (dq_is_phased<D, MASK>(p)) {
             const dim3 grid(p.B * p.H * (p.S / 256)), block(512);
-            if constexpr (D == 64) {
+            if constexpr (D == 64 || CAUSAL) {
                 if (p.thr8 > 0) {
                     if (with_delta) hipLaunchKernelGGL((mfma_dq_phased_kernel<T, D, CAUSAL, true, true>), grid, block, 0, stream, p);
                     else hipLaunchKernelGGL((mfma_dq_phased_kernel<T, D, CAUSAL, true, false>), grid, block, 0, stream, p);
