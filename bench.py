@@ -27,9 +27,9 @@ HBM_PEAK_GBS = 8000.0
 # (see profiles/); None where not measured.
 MEASURED_TRAFFIC = {
     # (workload, kernel): bytes read + written per launch (profiles/c3_hbm_traffic.txt)
-    ("C3", "fwd"): int((143.6 + 32.5) * 2**20),
-    ("C3", "bwd_dkdv"): int((210.7 + 64.0) * 2**20),
-    ("C3", "bwd_dq"): int((246.4 + 32.5) * 2**20),  # with the delta pre-pass folded in (reads O too)
+    ("C3", "fwd"): int((143.5 + 32.5) * 2**20),
+    ("C3", "bwd_dkdv"): int((211.6 + 64.0) * 2**20),
+    ("C3", "bwd_dq"): int((246.0 + 32.5) * 2**20),  # with the delta pre-pass folded in (reads O too)
     ("C3", "bwd_delta"): int((64.0 + 0.5) * 2**20),
 }
 
