@@ -175,14 +175,14 @@ def cpu_baseline(w, reps=3):
     if mask is not None:
         mask = mask.to(w.dtype)
     times = []
-    for rep in range(reps + 1):
+    for rep in range(max(reps, 1) + (1 if reps > 0 else 0)):
         tq, tk, tv = [x.clone().requires_grad_(w.backward) for x in (q, k, v)]
         t0 = time.perf_counter()
         out = oracle.sdpa_cpu(tq, tk, tv, mask, w.dropout_p, w.is_causal)
         if w.backward:
             out.backward(d_o)
         dt = time.perf_counter() - t0
-        if rep > 0:
+        if rep > 0 or reps == 0:
             times.append(dt)
     times.sort()
     med = times[len(times) // 2]
@@ -192,9 +192,95 @@ def cpu_baseline(w, reps=3):
         "cores": torch.get_num_threads(),
         "kind": "port",
         "sample": f"torch CPU scaled_dot_product_attention, full {w.name} workload "
-                  f"({'fwd+bwd' if w.backward else 'fwd'}), 1 warm-up + {reps} timed reps, median {med:.3f} s; "
+                  f"({'fwd+bwd' if w.backward else 'fwd'}), {'1 warm-up + ' + str(reps) + ' timed reps' if reps else 'one cold rep'}, median {med:.3f} s; "
                   f"os.cpu_count()={os.cpu_count()}",
     }
+
+
+def config_figures(dev, with_cpu):
+    """Forward and forward+backward figures of all five configurations (each with its own CPU baseline)."""
+    from trident_amd import workloads
+
+    out = {}
+    for name, wl in workloads.WORKLOADS.items():
+        pth = Path(wl, dev)
+        ms, pk = run_steps(pth, 3 if name == "C5" else 10, 2)
+        peak = PEAK_TFLOPS[_dtype_name(wl.dtype)]
+        f = wl.flops() / pk["fwd"] / 1e9
+        row = {"workload": describe(wl), "fwd_tflops": round(f, 2), "fwd_frac_of_peak": round(f / peak, 4),
+               "peak_tflops": peak, "kernel_ms": {k: round(v, 5) for k, v in pk.items()}}
+        if wl.backward:
+            t = wl.flops(True) / ms / 1e9
+            row.update(fwdbwd_tflops=round(t, 2), fwdbwd_frac_of_peak=round(t / peak, 4), ms_per_step=round(ms, 5))
+        if "bwd_delta" in pk:  # HBM-bound pre-pass: bytes it must move / its duration
+            gbs = pth.algorithmic_bytes("bwd_delta") / pk["bwd_delta"] / 1e6
+            row["delta_prepass"] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                    "frac": round(gbs / HBM_PEAK_GBS, 4)}
+        if wl.masked:  # mask streaming: every head reads its batch's S x S fp32 mask once per kernel
+            B, H, S, _ = pth.q.shape
+            logical, unique = 4.0 * B * H * S * S, 4.0 * B * S * S
+            row["mask_stream"] = {k: {"logical_GBps": round(logical / pk[k] / 1e6, 1),
+                                      "unique_GBps": round(unique / pk[k] / 1e6, 1)} for k in pk if k != "bwd_delta"}
+            row["mask_stream"]["note"] = ("fp32 mask bytes every workgroup asks for (logical: B*H*S*S*4; unique: "
+                                          "B*S*S*4, the heads of a batch share it) / kernel duration; HBM peak 8000 GB/s")
+        if with_cpu:
+            cb = cpu_baseline(wl, reps={"C3": 1, "C4": 1, "C5": 0}.get(name, 3))
+            row.update(cpu_tflops=cb["value"], cpu_cores=cb["cores"])
+        out[name] = row
+        del pth
+    return out
+
+
+def ceiling(dev):
+    """What the matrix pipe sustains on this box, in this process: MFMA-only loops on random operands (registers;
+    A operands from LDS; every LDS read feeding two MFMAs), a large bf16 GEMM, and the three C3 attention kernels."""
+    import torch
+
+    from trident_amd import _lib, workloads
+
+    lib = _lib.lib()
+    peak = PEAK_TFLOPS["bf16"]
+    res = {"peak_tflops": peak, "operands": "bf16 N(0,1) random (torch.randn, seed 1)"}
+    torch.manual_seed(1)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    operands = torch.randn(16 * 512 * 8, device=dev).to(torch.bfloat16)
+    out = torch.empty(cus * 512, device=dev, dtype=torch.float32)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+
+    def timed(fn, reps):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        ev[0].record()
+        for _ in range(reps):
+            fn()
+        ev[1].record()
+        torch.cuda.synchronize()
+        return ev[0].elapsed_time(ev[1]) / reps
+
+    iters = 4000
+    for mode, name in ((0, "mfma_registers"), (1, "mfma_lds_1_read_per_mfma"), (2, "mfma_lds_1_read_per_2_mfma")):
+        ms = timed(lambda: _lib.check(lib.tri_attn_probe_mfma(mode, cus, iters, operands.data_ptr(), out.data_ptr(),
+                                                               torch.cuda.current_stream().cuda_stream)), 5)
+        tf = cus * 8 * iters * 64 * 32768.0 / ms / 1e9
+        res[name] = {"ms": round(ms, 3), "tflops": round(tf, 1), "frac_of_peak": round(tf / peak, 4),
+                     "busy_x_clock_GHz": round(2.4 * tf / peak, 3)}
+    n = 8192
+    a = torch.randn(n, n, device=dev).to(torch.bfloat16)
+    b = torch.randn(n, n, device=dev).to(torch.bfloat16)
+    ms = timed(lambda: torch.matmul(a, b), 20)
+    tf = 2.0 * n**3 / ms / 1e9
+    res["torch_matmul_8192_bf16"] = {"ms": round(ms, 3), "tflops": round(tf, 1), "frac_of_peak": round(tf / peak, 4)}
+    del a, b
+    pth = Path(workloads.WORKLOADS["C3"], dev)
+    _, pk = run_steps(pth, 30, 5)
+    executed = {"fwd": 4.0 * 36 / 32, "bwd_dq": 6.0, "bwd_dkdv": 8.0 * 34 / 32}  # units of B H S^2 D / 2 the kernels run
+    unit = pth.w.flops() / 4.0
+    res["c3_kernels"] = {k: {"ms": round(v, 4), "credited_tflops": round(pth.algorithmic_flops(k) / v / 1e9, 1),
+                             "executed_tflops": round(executed[k] * unit / v / 1e9, 1),
+                             "executed_frac_of_peak": round(executed[k] * unit / v / 1e9 / peak, 4)}
+                        for k, v in pk.items() if k in executed}
+    return res
 
 
 def describe(w):
@@ -211,6 +297,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="C3")
     ap.add_argument("--report", action="store_true", help="also print all five configurations on stderr")
+    ap.add_argument("--no-configs", action="store_true", help="leave the five-configuration table out of the JSON line")
+    ap.add_argument("--ceiling", action="store_true",
+                    help="instead of the benchmark: print one JSON line with the MFMA ceiling of this box (random-operand "
+                         "MFMA loops, a bf16 GEMM, the C3 kernels)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (known HBM traffic) so that rocprofv3 FETCH_SIZE / "
@@ -228,6 +318,9 @@ def main():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
     w = workloads.WORKLOADS[a.workload]
+    if a.ceiling:
+        print(json.dumps({"ceiling": ceiling(dev)}), flush=True)
+        return
     if a.copy_calibration:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
         dst = torch.empty_like(src)
@@ -257,7 +350,8 @@ def main():
         "avg_launch_ms": round(per_kernel[dominant], 5),
     }
     result = {
-        "metric": "attention fwd & fwd+bwd TFLOP/s + % MFMA peak, bf16 causal S=4096 D=128",
+        "metric": ("attention fwd & fwd+bwd TFLOP/s + % MFMA peak, bf16 causal S=4096 D=128" if w.name == "C3" else
+                   "attention " + ("fwd+bwd" if w.backward else "fwd") + " TFLOP/s + % MFMA peak, " + describe(w)),
         "value": round(value, 1),
         "unit": "TFLOP/s",
         "n_gpus": 1,
@@ -287,6 +381,8 @@ def main():
                               "note": "same step through function.scaled_dot_product_attention + autograd"}
     if not a.no_cpu:
         result["cpu_baseline"] = cpu_baseline(w)
+    if not a.no_configs:
+        result["configs"] = config_figures(dev, not a.no_cpu)
     print(json.dumps(result), flush=True)
 
     if a.report:

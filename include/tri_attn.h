@@ -18,10 +18,15 @@
  *   - lse and delta are dense fp32 [B, H, S]. lse holds log2(sum_j exp(s_ij)) with
  *     s = q k^T * softmax_scale + mask, i.e. natural-log LSE times log2(e)
  *     (the same log2-domain statistic the reference saves, trident/kernel/attention.py:164,
- *     but always fp32).
+ *     but always fp32). For fp16/bf16 problems the matrix-core kernels sum the probabilities as rounded to
+ *     that type (the values that multiply V), so lse is accurate to half an ulp of the type times log2(e)
+ *     (2.8e-3 for bf16, 3.5e-4 for fp16), not to fp32 precision; the backward calls expect this very lse.
  *   - mask is additive, dtype mask_dtype, logical shape [B, H, S, S] with element strides;
  *     a stride of 0 broadcasts that dimension; the innermost mask stride must be 1.
  *     mask and is_causal are mutually exclusive (trident/operation/attention.py:41-43).
+ *   - A query row whose keys are ALL masked (-inf) behaves as in softmax: its output row and lse are NaN / -inf,
+ *     and in the backward its probabilities are NaN, which makes its dQ row and all of that head's dK and dV
+ *     NaN (what the reference's kernel and torch's attention give as well).
  *   - Causal rule: key j is visible to query i iff i >= j (trident/kernel/attention.py:131-134).
  *   - Dropout acts on the probabilities: P is multiplied by keep/(1 - thr8/256) where
  *     thr8 = clamp(rint(dropout_p * 256), 0, 256) and keep comes from Philox4x32-10:
@@ -29,8 +34,9 @@
  *       u8 = (r[i & 3] >> (8 * (j & 3))) & 0xff; keep = u8 >= thr8.
  *     The backward calls must be given the same seed, offset and dropout_p as the forward.
  *   - All entry points return 0 on success, a negative TRI_ATTN_E* code for an argument
- *     error, or a positive hipError_t if a launch failed. They are re-entrant and keep no
- *     mutable global state.
+ *     error, or a positive hipError_t if a launch failed. They are re-entrant; the only
+ *     state the library keeps is, per GPU, its compute-unit count (asked once, sizes the persistent
+ *     launches).
  */
 #ifndef TRI_ATTN_H
 #define TRI_ATTN_H
@@ -41,7 +47,7 @@
 extern "C" {
 #endif
 
-#define TRI_ATTN_ABI_VERSION 1
+#define TRI_ATTN_ABI_VERSION 2
 
 enum {
     TRI_ATTN_F32 = 0,
@@ -146,6 +152,13 @@ int tri_attn_bwd(const TriAttnArgs* args);
 int tri_attn_dropout_mask(uint64_t seed, uint64_t offset, float dropout_p, uint32_t bh,
                           int32_t row0, int32_t rows, int32_t col0, int32_t cols,
                           uint8_t* keep, void* stream);
+
+/* Calibration helper with no counterpart in the reference: `workgroups` workgroups of 512 threads each run
+ * iters x 64 bf16 32x32x16 MFMAs per wave on the caller's operand bits (operands: 16 * 512 * 16 bytes of
+ * device memory read as bf16 values, e.g. random normals; out: workgroups * 512 floats).
+ * mode 0: operands in registers; 1: every A operand read from LDS; 2: every LDS read feeds two MFMAs.
+ * Flops per launch = workgroups * 8 * iters * 64 * 32768. Used by bench.py --ceiling. */
+int tri_attn_probe_mfma(int mode, int workgroups, int iters, const void* operands, float* out, void* stream);
 
 #ifdef __cplusplus
 }

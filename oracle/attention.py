@@ -136,6 +136,46 @@ def attention_backward(q, k, v, d_out, mask=None, dropout_p=0.0, is_causal=False
     return dq, dk, dv, dmask, delta
 
 
+def attention_rows(q_rows, k, v, d_out_rows, row0, bh, mask_rows=None, dropout_p=0.0, is_causal=False, scale=None,
+                   seed=0, offset=0, o_rows=None):
+    """One head, the block of query rows [row0, row0 + R): everything that is local to those rows, so that a
+    full-size problem can be checked block by block (same formulas as attention_forward / attention_backward).
+    q_rows, d_out_rows: [R,D]; k, v: [S,D]; mask_rows: [R,S] or None; bh = b * H + h (dropout counter).
+    Returns dict(o [R,D], lse2 [R], delta [R], dq [R,D], dk_part [S,D], dv_part [S,D]) plus the sums of
+    absolute terms a_o, a_dq, a_dk_part, a_dv_part (see operand_abs_sums); dk_part / dv_part are
+    these rows' contributions to dK / dV. Under a causal mask the rows of a block that ends at S are the only
+    ones that see keys >= row0, so dk_part[row0:] and dv_part[row0:] are then the complete gradients."""
+    q_rows, k, v, d_out_rows = [np.asarray(x, dtype=np.float64) for x in (q_rows, k, v, d_out_rows)]
+    R, D = q_rows.shape
+    S = k.shape[0]
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    s = (q_rows @ k.T) * scale
+    rows = np.arange(row0, row0 + R)
+    if is_causal:
+        s = np.where(rows[:, None] >= np.arange(S)[None, :], s, -np.inf)
+    elif mask_rows is not None:
+        s = s + np.asarray(mask_rows, dtype=np.float64)
+    p, lse = _softmax_rows(s)
+    pz = p
+    z = None
+    if dropout_p > 0.0 and philox.dropout_threshold(dropout_p) != 0:
+        z = philox.dropout_keep_mask(seed, offset, bh, rows, np.arange(S), dropout_p).astype(np.float64)
+        z *= philox.dropout_scale(dropout_p)
+        pz = p * z
+    o = pz @ v
+    o_used = o if o_rows is None else np.asarray(o_rows, dtype=np.float64)
+    dlt = np.sum(d_out_rows * o_used, axis=-1)
+    dp = d_out_rows @ v.T
+    if z is not None:
+        dp = dp * z
+    ds = p * (dp - dlt[:, None])
+    ads = np.abs(ds)
+    return dict(o=o, lse2=lse * LOG2E, delta=dlt, dq=scale * (ds @ k), dk_part=scale * (ds.T @ q_rows),
+                dv_part=pz.T @ d_out_rows, a_o=pz @ np.abs(v), a_dq=scale * (ads @ np.abs(k)),
+                a_dk_part=scale * (ads.T @ np.abs(q_rows)), a_dv_part=pz.T @ np.abs(d_out_rows))
+
+
 def operand_abs_sums(q, k, v, d_out, mask=None, dropout_p=0.0, is_causal=False, scale=None, seed=0, offset=0, o=None):
     """Sum of |terms| of the contractions whose left operand a 16-bit matrix-core kernel must round
     (P for O and dV, dS for dQ and dK): A_O = |PZ| |V|, A_dV = |PZ|^T |dO|, A_dQ = scale |dS| |K|,

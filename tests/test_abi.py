@@ -89,6 +89,31 @@ def test_no_cpu_fallback():
         trident.function.scaled_dot_product_attention(x, x, x)
 
 
+def test_mixed_devices_raise_before_the_library_is_called():
+    """A host (or other-device) key, value, mask, grad_output, output or LSE must raise in Python: the
+    kernels would dereference its pointer on the GPU."""
+    from trident_amd import operation
+
+    cpu = torch.zeros(1, 1, 8, 16)
+    gpu0, gpu1 = torch.device("cuda:0"), torch.device("cuda:1")
+    for name in ("key", "value", "mask", "grad_output", "output", "log_sum_exp"):
+        with pytest.raises(RuntimeError, match=name + " is on cpu"):
+            operation._require_same_gpu(gpu0, **{name: cpu})
+    meta = torch.zeros(1, 1, 8, 16, device="meta")
+    with pytest.raises(RuntimeError, match="GPU only"):
+        operation._require_same_gpu(meta.device, key=meta)
+    operation._require_same_gpu(gpu0, key=None, mask=None)
+
+    class FakeCuda:  # stands for a tensor on another GPU (none exists on a CPU-only host)
+        device = gpu1
+
+    with pytest.raises(RuntimeError, match="value is on cuda:1, expected cuda:0"):
+        operation._require_same_gpu(gpu0, value=FakeCuda())
+    # through the operator: query on one device type, key on another
+    with pytest.raises(RuntimeError):
+        trident.function.scaled_dot_product_attention(meta, cpu, cpu)
+
+
 def test_api_surface():
     import inspect
 

@@ -322,3 +322,47 @@ def test_backward_with_saved_output_and_abs_sums():
     # non-negative inputs make the bound tight for O
     o_pos, _ = oracle.attention_forward(q, k, np.abs(v), is_causal=True)
     np.testing.assert_allclose(o_pos, a_o, atol=1e-13)
+
+
+# ---------------------------------------------------------------- row-block form (full-size checks)
+@pytest.mark.parametrize("variant", ["causal+dropout", "mask", "plain"])
+def test_row_blocks_reassemble_to_autograd_of_the_explicit_formula(variant):
+    """oracle.attention_rows against torch autograd of softmax(QK^T*scale + mask) * Z @ V: O, LSE, delta and dQ of
+    a block are the rows of the whole result; the dK/dV parts of all blocks add up to dK/dV; and under the
+    causal mask the LAST block alone gives dK/dV of its own keys."""
+    H, S, D, R = 2, 48, 8, 16
+    q, k, v, d_o = [_rand((1, H, S, D), s) for s in (11, 12, 13, 14)]
+    causal = variant.startswith("causal")
+    p, seed, offset = (0.3, 99, 2) if "dropout" in variant else (0.0, 0, 0)
+    mask = _rand((1, H, S, S), 15) if variant == "mask" else None
+    for h in range(H):
+        tq, tk, tv = [torch.tensor(x[0, h], requires_grad=True) for x in (q, k, v)]
+        s = tq @ tk.T / math.sqrt(D)
+        if causal:
+            s = s.masked_fill(~torch.ones(S, S, dtype=torch.bool).tril(), float("-inf"))
+        if mask is not None:
+            s = s + torch.tensor(mask[0, h])
+        pr = torch.softmax(s, -1)
+        if p > 0:
+            pr = pr * torch.tensor(philox.dropout_keep_mask(seed, offset, h, np.arange(S), np.arange(S), p) *
+                                   philox.dropout_scale(p))
+        out = pr @ tv
+        out.backward(torch.tensor(d_o[0, h]))
+        dk_sum, dv_sum = np.zeros((S, D)), np.zeros((S, D))
+        for r0 in range(0, S, R):
+            blk = oracle.attention_rows(q[0, h, r0:r0 + R], k[0, h], v[0, h], d_o[0, h, r0:r0 + R], r0, h,
+                                        mask_rows=None if mask is None else mask[0, h, r0:r0 + R], dropout_p=p,
+                                        is_causal=causal, seed=seed, offset=offset)
+            np.testing.assert_allclose(blk["o"], out.detach().numpy()[r0:r0 + R], rtol=0, atol=1e-12)
+            np.testing.assert_allclose(blk["lse2"], torch.logsumexp(s, -1).detach().numpy()[r0:r0 + R] * oracle.LOG2E,
+                                       rtol=0, atol=1e-12)
+            np.testing.assert_allclose(blk["delta"], (d_o[0, h] * out.detach().numpy()).sum(-1)[r0:r0 + R], rtol=0,
+                                       atol=1e-12)
+            np.testing.assert_allclose(blk["dq"], tq.grad.numpy()[r0:r0 + R], rtol=0, atol=1e-11)
+            dk_sum += blk["dk_part"]
+            dv_sum += blk["dv_part"]
+        np.testing.assert_allclose(dk_sum, tk.grad.numpy(), rtol=0, atol=1e-11)
+        np.testing.assert_allclose(dv_sum, tv.grad.numpy(), rtol=0, atol=1e-11)
+        if causal:
+            np.testing.assert_allclose(blk["dk_part"][S - R:], tk.grad.numpy()[S - R:], rtol=0, atol=1e-11)
+            np.testing.assert_allclose(blk["dv_part"][S - R:], tv.grad.numpy()[S - R:], rtol=0, atol=1e-11)

@@ -5,7 +5,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtrident_attn.so")
 ENOFUSE = -9  # tri_attn_bwd_dq_delta: no fused kernel for this problem, nothing launched
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _i64x4 = ctypes.c_int64 * 4
 
@@ -60,6 +60,7 @@ EXPORTS = (
     "tri_attn_bwd_dq_delta",
     "tri_attn_bwd",
     "tri_attn_dropout_mask",
+    "tri_attn_probe_mfma",
 )
 
 _lib = None
@@ -91,6 +92,9 @@ def lib():
             ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
             ctypes.c_void_p, ctypes.c_void_p,
         ]
+        cdll.tri_attn_probe_mfma.restype = ctypes.c_int
+        cdll.tri_attn_probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                             ctypes.c_void_p, ctypes.c_void_p]
         if cdll.tri_attn_version() != ABI_VERSION:
             raise RuntimeError("libtrident_attn.so ABI version mismatch: rebuild it")
         _lib = cdll

@@ -80,9 +80,11 @@ __global__ __launch_bounds__(256) void generic_fwd_kernel(const KParams p) {
 
     const int part = threadIdx.x & 3;
     const int r = threadIdx.x >> 2;
-    const int bh = blockIdx.y;
+    // one workgroup per (head, 64-row tile), head-major in grid.x (grid.y stops at 65 535)
+    const int tiles = (p.S + kRows - 1) / kRows;
+    const int bh = blockIdx.x / tiles;
     const int b = bh / p.H, h = bh % p.H;
-    const int row0 = blockIdx.x * kRows;
+    const int row0 = (blockIdx.x % tiles) * kRows;
     const int row = row0 + r;
     const bool row_ok = row < p.S;
     const int row_c = row_ok ? row : p.S - 1;
@@ -153,9 +155,11 @@ __global__ __launch_bounds__(256) void generic_dq_kernel(const KParams p) {
 
     const int part = threadIdx.x & 3;
     const int r = threadIdx.x >> 2;
-    const int bh = blockIdx.y;
+    // one workgroup per (head, 64-row tile), head-major in grid.x (grid.y stops at 65 535)
+    const int tiles = (p.S + kRows - 1) / kRows;
+    const int bh = blockIdx.x / tiles;
     const int b = bh / p.H, h = bh % p.H;
-    const int row0 = blockIdx.x * kRows;
+    const int row0 = (blockIdx.x % tiles) * kRows;
     const int row = row0 + r;
     const bool row_ok = row < p.S;
     const int row_c = row_ok ? row : p.S - 1;
@@ -187,7 +191,7 @@ __global__ __launch_bounds__(256) void generic_dq_kernel(const KParams p) {
             float x = quad_sum(dot_slice<D>(q, sK + u * D, part)) * p.scale_log2;
             float dp = quad_sum(dot_slice<D>(g, sV + u * D, part));
             if (p.mask && j < p.S) x = fmaf(load_mask_elem(p.mask, p.mask_dtype, mrow + j), kLog2e, x);
-            const bool visible = j < p.S && (!p.causal || j <= row) && x != -INFINITY;
+            const bool visible = j < p.S && (!p.causal || j <= row);
             const float pr = visible ? fast_exp2(x - lse) : 0.f;
             if (p.thr8 > 0) dp = dropout_keep(p, bh, row, j) ? dp * p.zscale : 0.f;
             const float ds = pr * (dp - dlt);
@@ -213,9 +217,11 @@ __global__ __launch_bounds__(256) void generic_dkdv_kernel(const KParams p) {
 
     const int part = threadIdx.x & 3;
     const int r = threadIdx.x >> 2;
-    const int bh = blockIdx.y;
+    // one workgroup per (head, 64-row tile), head-major in grid.x (grid.y stops at 65 535)
+    const int tiles = (p.S + kRows - 1) / kRows;
+    const int bh = blockIdx.x / tiles;
     const int b = bh / p.H, h = bh % p.H;
-    const int col0 = blockIdx.x * kRows;
+    const int col0 = (blockIdx.x % tiles) * kRows;
     const int col = col0 + r;
     const bool col_ok = col < p.S;
     const int col_c = col_ok ? col : p.S - 1;
@@ -249,7 +255,7 @@ __global__ __launch_bounds__(256) void generic_dkdv_kernel(const KParams p) {
             float x = quad_sum(dot_slice<D>(k, sQ + u * D, part)) * p.scale_log2;
             float dp = quad_sum(dot_slice<D>(v, sG + u * D, part));
             if (p.mask && i < p.S) x = fmaf(load_mask_elem(p.mask, p.mask_dtype, mbase + i * p.ms[2]), kLog2e, x);
-            const bool visible = i < p.S && col_ok && (!p.causal || col <= i) && x != -INFINITY;
+            const bool visible = i < p.S && col_ok && (!p.causal || col <= i);
             float pr = visible ? fast_exp2(x - sLse[u]) : 0.f;
             if (p.thr8 > 0) {
                 const bool keep = dropout_keep(p, bh, i, col);
@@ -300,7 +306,9 @@ __global__ __launch_bounds__(256) void generic_delta_kernel(const KParams p) {
 template <typename T, int D>
 int launch_generic(int which, const KParams& p, hipStream_t stream) {
     const dim3 block(256);
-    const dim3 grid((p.S + kRows - 1) / kRows, p.B * p.H);
+    const int64_t groups = static_cast<int64_t>((p.S + kRows - 1) / kRows) * p.B * p.H;
+    if (groups > 2147483647LL) return TRI_ATTN_ESHAPE;
+    const dim3 grid(static_cast<unsigned>(groups));
     switch (which) {
         case kGenericFwd:
             hipLaunchKernelGGL((generic_fwd_kernel<T, D>), grid, block, 0, stream, p);

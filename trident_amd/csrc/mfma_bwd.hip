@@ -78,7 +78,6 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
         gf[kk] = *reinterpret_cast<const u32x4*>(gorowp + (2 * kk + h) * 16);
     }
     float lse = p.lse[static_cast<int64_t>(bh) * p.S + qrow];
-    if (lse == -INFINITY) lse = INFINITY;  // fully masked row: every probability is 0
     const float dlt = p.delta[static_cast<int64_t>(bh) * p.S + qrow];
     const float c = p.scale_log2;
 
@@ -415,7 +414,6 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
     TRI_WAIT_VMCNT(0);
     settle(lse);
     if constexpr (!DELTA) settle(dlt);
-    if (lse == -INFINITY) lse = INFINITY;  // fully masked row: every probability is 0
     lds_barrier();
     if (n_first > 1) issue_tile(1);
     if (n_first > 2) issue_tile(2);
@@ -693,10 +691,6 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
                 for (int g = 0; g < 4; ++g) {
                     f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + 32 * qb + 8 * g + 4 * h);
                     const f32x4 d4 = *reinterpret_cast<const f32x4*>(sDelta + 32 * qb + 8 * g + 4 * h);
-                    if constexpr (MASK != kNoMask) {
-#pragma unroll
-                        for (int bb = 0; bb < 4; ++bb) l4[bb] = l4[bb] == -INFINITY ? INFINITY : l4[bb];
-                    }
                     uint32_t dw[4];
                     if constexpr (DROPOUT) {
                         const Philox4 r = quad_bcast_from(g, mine);  // lane g of the quad generated rows rb + 8 g + 4 h .. +3
@@ -1012,10 +1006,6 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
                     const int g = 2 * gg + g2;
                     f32x4 l4 = sc_lse[g];
                     const f32x4 d4 = dlt4[g2];
-                    if constexpr (MASK != kNoMask) {
-#pragma unroll
-                        for (int bb = 0; bb < 4; ++bb) l4[bb] = l4[bb] == -INFINITY ? INFINITY : l4[bb];
-                    }
                     uint32_t dw[4];
                     if constexpr (DROPOUT) {
                         const Philox4 r = quad_bcast_from(g, mine);  // lane g of the quad generated rows rb + 8 g + 4 h .. +3

@@ -65,6 +65,8 @@ bool mfma_supported(int which, int dtype, const KParams& p) {
     }
     switch (which) {
         case kMfmaFwd:
+            // K and V tiles are fetched by LDS-direct loads with 32-bit per-lane byte offsets
+            if (!tile_offsets_fit(p.ks) || !tile_offsets_fit(p.vs)) return false;
             return aligned16(p.o) && strides8(p.os);
         case kMfmaDkdv:
             // the streamed tiles are addressed with 32-bit byte offsets from a per-tile base
@@ -72,7 +74,8 @@ bool mfma_supported(int which, int dtype, const KParams& p) {
             return aligned16(p.d_o) && strides8(p.dos) && aligned16(p.dk) && strides8(p.dks) && aligned16(p.dv) &&
                    strides8(p.dvs);
         case kMfmaDq:
-            if (!tile_offsets_fit(p.ks) || !tile_offsets_fit(p.vs)) return false;
+            // (K, V tiles; the phased kernel also stages its Q, dO and O rows that way)
+            if (!tile_offsets_fit(p.ks) || !tile_offsets_fit(p.vs) || !tile_offsets_fit(p.qs) || !tile_offsets_fit(p.dos)) return false;
             // the mask gradient is written by the generic dQ kernel
             return p.dmask == nullptr && aligned16(p.d_o) && strides8(p.dos) && aligned16(p.dq) && strides8(p.dqs);
         default:
@@ -84,7 +87,7 @@ bool mfma_supported(int which, int dtype, const KParams& p) {
 bool mfma_dq_fuses_delta(const KParams& p) {
     if (p.mask != nullptr || p.S % 256 != 0) return false;
     if (!(p.D == 64 || p.thr8 <= 0 || p.causal)) return false;  // (the phased dQ kernel's own limits)
-    return aligned16(p.o) && strides8(p.os);
+    return aligned16(p.o) && strides8(p.os) && tile_offsets_fit(p.os);
 }
 
 int persistent_grid(int items) {

@@ -1,0 +1,86 @@
+// Calibration kernels: what the matrix pipe of this GPU sustains on random operands, alone and with its A
+// operands streamed from LDS. They have no counterpart in the reference; bench.py --ceiling times them next
+// to a large bf16 GEMM and the attention kernels, so that an attention kernel's distance from the published
+// MFMA peak can be split into "cycles not spent in MFMAs" and "clock below 2.4 GHz under this load".
+#include "launch.hpp"
+#include "mfma_common.hpp"
+
+namespace tri {
+namespace {
+
+constexpr int kProbeThreads = 512;      // 8 waves per workgroup, two per SIMD
+constexpr int kProbeLdsBytes = 128 * 1024;  // a wave's reads of one loop trip span 64 KiB from a base that moves per trip
+
+// MODE 0: operands in registers (8 A and 8 B fragments per wave, all pairings over 8 loop trips)
+// MODE 1: every MFMA takes its A fragment from LDS (one ds_read_b128 per MFMA, as the attention kernels do)
+// MODE 2: every A fragment read from LDS feeds two MFMAs (two B fragments, two accumulators)
+template <int MODE>
+__global__ __launch_bounds__(kProbeThreads) void probe_kernel(const u32x4* __restrict__ operands, float* out, int iters) {
+    __shared__ __attribute__((aligned(1024))) char smem[MODE == 0 ? 16 : kProbeLdsBytes];
+    const int tid = threadIdx.x, lane = tid & 63;
+    u32x4 a[8], b[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        a[i] = operands[i * kProbeThreads + tid];
+        b[i] = operands[(8 + i) * kProbeThreads + tid];
+    }
+    if constexpr (MODE != 0) {
+        for (int i = tid; i < kProbeLdsBytes / 16; i += kProbeThreads)
+            *reinterpret_cast<u32x4*>(smem + i * 16) = operands[i % (16 * kProbeThreads)];
+        __syncthreads();
+    }
+    f32x16 c[4] = {zero16(), zero16(), zero16(), zero16()};
+    // the LDS modes keep a ring of 8 fragments in flight across loop trips (the base moves per trip, so no read
+    // can be hoisted out of the loop)
+    auto base_of = [&](int it) { return smem + (((it + (tid >> 6) * 8) & 63) << 10) + lane * 16; };
+    u32x4 ring[8];
+    if constexpr (MODE != 0) {
+#pragma unroll
+        for (int r = 0; r < 8; ++r) ring[r] = lds_read16(base_of(0), r * 1024);
+    }
+    for (int it = 0; it < iters; ++it) {
+        if constexpr (MODE == 0) {
+#pragma unroll
+            for (int r = 0; r < 8; ++r)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) c[j & 3] = Mma<bf16_t>::run(a[j], b[(j + r) & 7], c[j & 3]);
+        } else {
+            constexpr int kReads = MODE == 1 ? 64 : 32;
+            const char* base = base_of(it);
+            const char* next = base_of(it + 1);
+#pragma unroll
+            for (int j = 0; j < kReads; ++j) {
+                const u32x4 f = ring[j & 7];
+                if constexpr (MODE == 1) {
+                    c[j & 3] = Mma<bf16_t>::run(f, b[j & 7], c[j & 3]);
+                } else {
+                    c[(2 * j) & 3] = Mma<bf16_t>::run(f, b[j & 7], c[(2 * j) & 3]);
+                    c[(2 * j + 1) & 3] = Mma<bf16_t>::run(f, b[(j + 3) & 7], c[(2 * j + 1) & 3]);
+                }
+                ring[j & 7] = j + 8 < kReads ? lds_read16(base, (j + 8) * 1024) : lds_read16(next, (j + 8 - kReads) * 1024);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s += (c[0][i] + c[1][i]) + (c[2][i] + c[3][i]);
+    out[static_cast<int64_t>(blockIdx.x) * kProbeThreads + tid] = s;
+}
+
+}  // namespace
+}  // namespace tri
+
+using namespace tri;
+
+extern "C" int tri_attn_probe_mfma(int mode, int workgroups, int iters, const void* operands, float* out, void* stream) {
+    if (operands == nullptr || out == nullptr) return TRI_ATTN_ENULL;
+    if (workgroups <= 0 || iters <= 0 || mode < 0 || mode > 2) return TRI_ATTN_ESHAPE;
+    const dim3 grid(workgroups), block(kProbeThreads);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const u32x4* ops = static_cast<const u32x4*>(operands);
+    if (mode == 0) hipLaunchKernelGGL(probe_kernel<0>, grid, block, 0, st, ops, out, iters);
+    else if (mode == 1) hipLaunchKernelGGL(probe_kernel<1>, grid, block, 0, st, ops, out, iters);
+    else hipLaunchKernelGGL(probe_kernel<2>, grid, block, 0, st, ops, out, iters);
+    return static_cast<int>(hipGetLastError());
+}

@@ -27,6 +27,17 @@ def _dense_rows(t: torch.Tensor) -> torch.Tensor:
     return t
 
 
+def _require_same_gpu(device, **tensors):
+    """Every tensor handed to the library must live on the one GPU the call runs on: the kernels
+    dereference the raw pointers, so a host or other-device tensor must stop here, as an exception."""
+    if device.type != "cuda":
+        raise RuntimeError("trident_amd attention runs on the GPU only; got a tensor on " + str(device))
+    for name, t in tensors.items():
+        if t is not None and t.device != device:
+            raise RuntimeError(f"trident_amd attention: {name} is on {t.device}, expected {device} "
+                               "(all tensors of a call must be on the same GPU)")
+
+
 def _next_seed():
     fixed = config.dropout_seed
     if fixed is None:
@@ -144,8 +155,7 @@ class Attention(torch.autograd.Function):
     def _forward(query, key, value, mask, dropout_p, is_causal, softmax_scale, seed, offset):
         assert query.shape[-1] == key.shape[-1] and key.shape[-1] == value.shape[-1]
         assert key.shape[-1] in {16, 32, 64, 128}
-        if not query.is_cuda:
-            raise RuntimeError("trident_amd attention runs on the GPU only; got a tensor on " + str(query.device))
+        _require_same_gpu(query.device, key=key, value=value, mask=mask)
         if key.shape != query.shape or value.shape != query.shape:
             raise ValueError("query, key and value must have the same shape.")
         if key.dtype != query.dtype or value.dtype != query.dtype:
@@ -173,7 +183,11 @@ class Attention(torch.autograd.Function):
 
     @staticmethod
     def _backward(grad_output, query, key, value, output, log2sum, mask, softmax_scale, dropout_p, is_causal,
-                  seed, offset, want_grad_mask):
+                  seed, offset, want_grad_mask, delta_out=None):
+        """``delta_out``: optional fp32 [B,H,S] tensor that receives delta (the backward's intermediate,
+        trident/operation/attention.py:155); allocated here when not given."""
+        _require_same_gpu(query.device, key=key, value=value, mask=mask, grad_output=grad_output, output=output,
+                          log_sum_exp=log2sum)
         lib = _lib.lib()
         query, key, value = _dense_rows(query), _dense_rows(key), _dense_rows(value)
         grad_output = _dense_rows(grad_output)
@@ -181,7 +195,7 @@ class Attention(torch.autograd.Function):
         grad_query = torch.empty(query.shape, device=query.device, dtype=query.dtype)
         grad_key = torch.empty(key.shape, device=key.device, dtype=key.dtype)
         grad_value = torch.empty(value.shape, device=value.device, dtype=value.dtype)
-        delta = torch.empty_like(log2sum)
+        delta = torch.empty_like(log2sum) if delta_out is None else delta_out
         full = (num_batches, num_heads, y_size, y_size)
         mask_view = _expand_mask(mask.detach(), full) if mask is not None else None
         grad_mask_full = torch.empty(full, device=mask.device, dtype=mask.dtype) if want_grad_mask else None
