@@ -36,7 +36,7 @@
  *   - All entry points return 0 on success, a negative TRI_ATTN_E* code for an argument
  *     error, or a positive hipError_t if a launch failed. They are re-entrant; the only
  *     state the library keeps is, per GPU, its compute-unit count (asked once, sizes the persistent
- *     launches).
+ *     launches) and the address of tri_attn_bwd_noalloc's buffer.
  */
 #ifndef TRI_ATTN_H
 #define TRI_ATTN_H
@@ -65,7 +65,8 @@ enum {
     TRI_ATTN_EDROPOUT = -6,   /* dropout_p outside [0,1] */
     TRI_ATTN_ESIZE = -7,      /* struct_size does not match this ABI version */
     TRI_ATTN_EALIGN = -8,     /* a pointer or stride breaks the 16-byte alignment the kernels need */
-    TRI_ATTN_ENOFUSE = -9     /* tri_attn_bwd_dq_delta only: no fused kernel serves this problem, nothing was launched */
+    TRI_ATTN_ENOFUSE = -9,    /* tri_attn_bwd_dq_delta only: no fused kernel serves this problem, nothing was launched */
+    TRI_ATTN_ESCRATCH = -10   /* tri_attn_bwd_noalloc only: B*H*S exceeds TRI_ATTN_NOALLOC_MAX_ROWS, nothing was launched */
 };
 
 typedef struct TriAttnArgs {
@@ -144,6 +145,17 @@ int tri_attn_bwd_dq_delta(const TriAttnArgs* args);
  * kernels and in another order: without a mask, for sequence lengths that are multiples of 256 (and
  * without dropout at D = 128) the dQ kernel computes delta on its way and runs before dK/dV. */
 int tri_attn_bwd(const TriAttnArgs* args);
+
+/* tri_attn_bwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc). It has no counterpart in the reference, whose backward allocates
+ * delta itself (trident/operation/attention.py:155). Same results as tri_attn_bwd on the same arguments,
+ * except that args->delta is ignored (it may be NULL): delta lives in a buffer inside the library,
+ * TRI_ATTN_NOALLOC_MAX_ROWS fp32 values (4 MiB) that every GPU the library runs on holds until the process
+ * ends. B*H*S above that limit returns TRI_ATTN_ESCRATCH and launches nothing. The call allocates and frees
+ * nothing. All calls on one GPU share that GPU's buffer: calls that may overlap on one GPU (different streams
+ * or threads) race on it and must be serialised by the caller; calls on one stream are ordered. */
+#define TRI_ATTN_NOALLOC_MAX_ROWS (1 << 20)
+int tri_attn_bwd_noalloc(const TriAttnArgs* args);
 
 /* Debug / parity helper with no counterpart in the reference (its dropout stream is unpinned):
  * writes the dropout keep decisions (1 = kept) for head index bh, rows [row0,row0+rows),

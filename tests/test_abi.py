@@ -60,6 +60,13 @@ def test_status_codes_without_gpu():
     assert lib.tri_attn_fwd(ctypes.byref(args)) == -5
     assert b"mask and is_causal" in lib.tri_attn_strerror(-5)
     assert lib.tri_attn_dropout_mask(0, 0, 0.1, 0, 0, 4, 0, 4, None, None) == -1
+    # the entry point that allocates nothing refuses problems beyond its buffer before it touches the GPU
+    big = _lib.TriAttnArgs()
+    big.struct_size = ctypes.sizeof(big)
+    big.dtype = 2
+    big.B, big.H, big.S, big.D = 1, 64, _lib.NOALLOC_MAX_ROWS // 64 + 128, 64
+    assert lib.tri_attn_bwd_noalloc(ctypes.byref(big)) == _lib.ESCRATCH
+    assert lib.tri_attn_bwd_noalloc(None) == -1
 
 
 def test_reference_value_errors():

@@ -6,6 +6,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtrident_attn.so")
 ENOFUSE = -9  # tri_attn_bwd_dq_delta: no fused kernel for this problem, nothing launched
 ABI_VERSION = 2
+ESCRATCH = -10  # tri_attn_bwd_noalloc: B*H*S above NOALLOC_MAX_ROWS, nothing launched
+NOALLOC_MAX_ROWS = 1 << 20
 
 _i64x4 = ctypes.c_int64 * 4
 
@@ -59,6 +61,7 @@ EXPORTS = (
     "tri_attn_bwd_dq",
     "tri_attn_bwd_dq_delta",
     "tri_attn_bwd",
+    "tri_attn_bwd_noalloc",
     "tri_attn_dropout_mask",
     "tri_attn_probe_mfma",
 )
@@ -82,7 +85,7 @@ def lib():
         cdll.tri_attn_strerror.restype = ctypes.c_char_p
         cdll.tri_attn_strerror.argtypes = [ctypes.c_int]
         for name in ("tri_attn_fwd", "tri_attn_bwd_delta", "tri_attn_bwd_dkdv", "tri_attn_bwd_dq",
-                     "tri_attn_bwd_dq_delta", "tri_attn_bwd"):
+                     "tri_attn_bwd_dq_delta", "tri_attn_bwd", "tri_attn_bwd_noalloc"):
             fn = getattr(cdll, name)
             fn.restype = ctypes.c_int
             fn.argtypes = [ctypes.POINTER(TriAttnArgs)]

@@ -2,8 +2,14 @@
 #include <math.h>
 #include <string.h>
 
+#include <atomic>
+
 #include "common.hpp"
 #include "launch.hpp"
+
+// Backward scratch of tri_attn_bwd_noalloc (see below): file scope, one copy per GPU. In host code this name is
+// only a stand-in for hipGetSymbolAddress; kernels get the device address as an argument.
+static __device__ __align__(256) float scratch[TRI_ATTN_NOALLOC_MAX_ROWS];
 
 namespace tri {
 namespace {
@@ -115,6 +121,31 @@ __global__ void dropout_mask_kernel(KParams p, uint32_t bh, int row0, int rows, 
     keep[n] = dropout_keep(p, bh, i, j) ? 1 : 0;
 }
 
+// ---- tri_attn_bwd_noalloc: the backward's delta buffer inside the library
+// delta (fp32 [B,H,S]) is the one piece of device memory the backward needs beyond its inputs and outputs: the
+// dQ kernel (or the delta pre-pass) writes it, the dK/dV kernel reads it. For callers that cannot allocate it
+// lives here, once per GPU, for the life of the process.
+constexpr int64_t kScratchRows = TRI_ATTN_NOALLOC_MAX_ROWS;
+constexpr int kMaxDevices = 64;
+std::atomic<float*> scratch_ptr[kMaxDevices];  // device address of `scratch` on each GPU (the name above is a host-side stand-in)
+
+// Address of this GPU's copy of `scratch`, asked once per device with that device current.
+int scratch_for_current_device(float** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (dev < 0 || dev >= kMaxDevices) return TRI_ATTN_ESHAPE;
+    float* ptr = scratch_ptr[dev].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
+        e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return static_cast<int>(e);
+        if (ptr == nullptr) return static_cast<int>(hipErrorInvalidSymbol);
+        scratch_ptr[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return TRI_ATTN_OK;
+}
+
 }  // namespace
 }  // namespace tri
 
@@ -136,6 +167,7 @@ const char* tri_attn_strerror(int status) {
         case TRI_ATTN_ESIZE: return "TriAttnArgs.struct_size does not match this library";
         case TRI_ATTN_EALIGN: return "pointer or stride alignment not supported";
         case TRI_ATTN_ENOFUSE: return "no fused dQ + delta kernel for this problem (nothing launched)";
+        case TRI_ATTN_ESCRATCH: return "tri_attn_bwd_noalloc: B*H*S exceeds TRI_ATTN_NOALLOC_MAX_ROWS (nothing launched)";
         default: break;
     }
     if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
@@ -195,6 +227,19 @@ int tri_attn_bwd(const TriAttnArgs* args) {
     rc = tri_attn_bwd_dkdv(args);
     if (rc) return rc;
     return tri_attn_bwd_dq(args);
+}
+
+int tri_attn_bwd_noalloc(const TriAttnArgs* args) {
+    if (args == nullptr) return TRI_ATTN_ENULL;
+    if (args->struct_size != sizeof(TriAttnArgs)) return TRI_ATTN_ESIZE;
+    if (args->B <= 0 || args->H <= 0 || args->S <= 0) return TRI_ATTN_ESHAPE;
+    if (static_cast<int64_t>(args->B) * args->H * args->S > kScratchRows) return TRI_ATTN_ESCRATCH;
+    TriAttnArgs a = *args;  // (host copy of a plain struct)
+    const int rc = scratch_for_current_device(&a.delta);
+    if (rc) return rc;
+    // every row of delta that dK/dV reads is written first by this call's dQ kernel or delta pre-pass:
+    // nothing of the previous call's contents needs clearing
+    return tri_attn_bwd(&a);
 }
 
 int tri_attn_dropout_mask(uint64_t seed, uint64_t offset, float dropout_p, uint32_t bh, int32_t row0, int32_t rows,
