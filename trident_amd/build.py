@@ -1,10 +1,16 @@
 """Builds libtrident_attn.so (the C-ABI library with the gfx950 kernels) in-tree with hipcc.
 
-    python -m trident_amd.build          # compile every csrc/*.hip and link
+    python -m trident_amd.build               # compile every csrc/*.hip and link
+    python -m trident_amd.build --resources   # also print the per-kernel register / LDS / scratch table
+
+Every build reads the compiler's kernel-resource-usage remarks and FAILS when a kernel that one of the five
+benchmark configurations launches uses scratch memory (spilled vector registers): a scratch reload is a
+vector-memory load, and the kernels' hand-counted vmcnt waits would then drain the tile prefetch on every reload.
 """
 import concurrent.futures
 import glob
 import os
+import re
 import subprocess
 import sys
 
@@ -22,35 +28,144 @@ FLAGS = [
     "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    "-Wno-pass-failed",  # 4-wave variants ask for two workgroups per CU and get one (LDS): known, not an error
     "-Wno-inline-asm",  # the LDS-direct load helpers name M0 as clobbered, which clang reports as a reserved register
     "-I", INCLUDE,
     "-I", CSRC,
+    "-Rpass-analysis=kernel-resource-usage",
 ]
+
+# The kernels the five benchmark configurations launch (demangled name without the parameter list).
+BASELINE_KERNELS = {
+    "mfma_fwd_kernel<_Float16, 64, 8, false, 0, false>": "C2 fwd",
+    "mfma_fwd_kernel<__bf16, 128, 8, true, 0, false>": "C3 fwd",
+    "mfma_dq_phased_kernel<__bf16, 128, true, false, true>": "C3 dQ + delta",
+    "mfma_dkdv_phased_kernel<__bf16, 128, true>": "C3 dK/dV",
+    "mfma_fwd_kernel<__bf16, 64, 8, false, 1, false>": "C4 fwd",
+    "delta_kernel<__bf16, 64>": "C4 delta",
+    "mfma_dkdv_wide_kernel<__bf16, 64, 8, false, 1, false>": "C4 dK/dV",
+    "mfma_dq_kernel<__bf16, 64, 8, false, 1, false>": "C4 dQ",
+    "mfma_fwd_kernel<__bf16, 128, 8, true, 0, true>": "C5 fwd",
+    "mfma_dq_phased_kernel<__bf16, 128, true, true, true>": "C5 dQ + delta",
+    "mfma_dkdv_pair_kernel<__bf16, 128, true, 0, true>": "C5 dK/dV",
+    "generic_fwd_kernel<float, 32>": "C1 fwd",
+}
+_FIELDS = [("TotalSGPRs", "sgpr"), ("VGPRs", "vgpr"), ("AGPRs", "agpr"), ("ScratchSize [bytes/lane]", "scratch"),
+           ("Occupancy [waves/SIMD]", "occupancy"), ("SGPRs Spill", "sgpr_spill"), ("VGPRs Spill", "vgpr_spill"),
+           ("LDS Size [bytes/block]", "lds")]
+
+
+def _parse_resources(stderr):
+    """{mangled kernel name: {field: int}} from the -Rpass-analysis=kernel-resource-usage remarks."""
+    out, cur = {}, None
+    for line in stderr.splitlines():
+        m = re.search(r"remark:\s+Function Name: (\S+)", line)
+        if m:
+            cur = out.setdefault(m.group(1), {})
+            continue
+        if cur is None:
+            continue
+        for label, key in _FIELDS:
+            m = re.search(r"remark:\s+" + re.escape(label) + r": (\d+)", line)
+            if m:
+                cur[key] = int(m.group(1))
+    return out
+
+
+def _demangle(names):
+    """Readable names of this library's kernels (tri::(anonymous)::name<type / int / bool arguments>(...))."""
+    out = {}
+    for n in names:
+        m = re.match(r"_ZN3tri12_GLOBAL__N_1(\d+)", n)
+        if not m:
+            out[n] = n
+            continue
+        ln = int(m.group(1))
+        name, rest = n[m.end():m.end() + ln], n[m.end() + ln:]
+        args = []
+        if rest.startswith("I"):
+            rest = rest[1:]
+            while rest and not rest.startswith("E"):
+                for pat, fn in ((r"DF16_", lambda g: "_Float16"), (r"DF16b", lambda g: "__bf16"), (r"f", lambda g: "float"),
+                                (r"Li(\d+)E", lambda g: g.group(1)), (r"Lb([01])E", lambda g: "true" if g.group(1) == "1" else "false")):
+                    g = re.match(pat, rest)
+                    if g:
+                        args.append(fn(g))
+                        rest = rest[g.end():]
+                        break
+                else:
+                    args, rest = ["?"], ""
+        out[n] = name + ("<" + ", ".join(args) + ">" if args else "")
+    return out
 
 
 def _compile(src):
     obj = os.path.join(OBJ_DIR, os.path.basename(src)[:-4] + ".o")
     cmd = [HIPCC, *FLAGS, "-c", src, "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
-    err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
+    lines, skip = [], 0
+    for l in res.stderr.splitlines():  # (a remark is followed by two lines quoting the source)
+        if "packed-fp32-ops" in l:
+            continue
+        if "-Rpass-analysis=kernel-resource-usage" in l:
+            skip = 2
+            continue
+        if skip and (re.match(r"\s*\d+ \|", l) or re.match(r"\s*\|", l)):
+            skip -= 1
+            continue
+        skip = 0
+        lines.append(l)
+    err = "\n".join(lines)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{err}")
     if err.strip():
         sys.stderr.write(err + "\n")
-    return obj
+    return obj, _parse_resources(res.stderr)
 
 
-def build(verbose=True):
+def resource_table(resources):
+    names = _demangle(sorted(resources))
+    rows = sorted((names[m], r) for m, r in resources.items())
+    head = f"{'kernel':<64} {'config':<14} {'VGPR':>5} {'AGPR':>5} {'SGPR':>5} {'SGPR spill':>10} {'VGPR spill':>10} " \
+           f"{'scratch B':>9} {'LDS B':>7} {'waves/SIMD':>10}"
+    out = [head]
+    for name, r in rows:
+        out.append(f"{name:<64} {BASELINE_KERNELS.get(name, ''):<14} {r.get('vgpr', 0):>5} {r.get('agpr', 0):>5} "
+                   f"{r.get('sgpr', 0):>5} {r.get('sgpr_spill', 0):>10} {r.get('vgpr_spill', 0):>10} {r.get('scratch', 0):>9} "
+                   f"{r.get('lds', 0):>7} {r.get('occupancy', 0):>10}")
+    return "\n".join(out)
+
+
+def check_baseline_kernels(resources):
+    names = _demangle(sorted(resources))
+    found = {names[m]: r for m, r in resources.items()}
+    missing = [k for k in BASELINE_KERNELS if k not in found]
+    if missing:
+        raise RuntimeError("kernels of the benchmark configurations not found in the build: " + ", ".join(missing))
+    bad = [f"{k} ({BASELINE_KERNELS[k]}): {found[k].get('scratch', 0)} bytes of scratch per lane"
+           for k in BASELINE_KERNELS if found[k].get("scratch", 0) > 0]
+    if bad:
+        raise RuntimeError("benchmark kernels spill vector registers to scratch:\n  " + "\n  ".join(bad))
+
+
+def build(verbose=True, resources=False):
     os.makedirs(OBJ_DIR, exist_ok=True)
     sources = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
-        objs = list(pool.map(_compile, sources))
+        results = list(pool.map(_compile, sources))
+    objs = [o for o, _ in results]
+    usage = {}
+    for _, r in results:
+        usage.update(r)
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", OUT, *objs]
     subprocess.check_call(cmd)
+    if resources:
+        print(resource_table(usage))
+    check_baseline_kernels(usage)
     if verbose:
-        print(f"built {OUT} from {len(sources)} sources")
+        print(f"built {OUT} from {len(sources)} sources; {len(usage)} kernels, none of the benchmark kernels uses scratch")
     return OUT
 
 
 if __name__ == "__main__":
-    build()
+    build(resources="--resources" in sys.argv[1:])

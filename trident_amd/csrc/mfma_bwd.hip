@@ -502,7 +502,11 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
         static_assert(NW * Store::kPatchBytes <= kStages * kStageBytes, "patches must fit into the ring");
         char* out0 = static_cast<char*>(p.dq) + (b * p.dqs[0] + hd * p.dqs[1] + static_cast<int64_t>(wrow0) * p.dqs[2]) * 2;
         const float sc = p.scale;
-        Store::run(acc, [sc](float x) { return x * sc; }, smem + wave * Store::kPatchBytes, out0, p.dqs[2] * 2, lane);
+        // the lane index taken afresh: the epilogue's per-lane offsets are then computed here instead of being
+        // kept (or, with every register in use, spilled) across the loop
+        int elane = threadIdx.x & 63;
+        asm volatile("" : "+v"(elane));
+        Store::run(acc, [sc](float x) { return x * sc; }, smem + wave * Store::kPatchBytes, out0, p.dqs[2] * 2, elane);
     }
 }
 
