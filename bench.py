@@ -231,6 +231,106 @@ def config_figures(dev, with_cpu):
     return out
 
 
+def sibling_ops(dev):
+    """HBM-bound sibling operations through the operator API on one large input (bf16, 16384 x 8192 = 256 MiB):
+    achieved bytes/s against the 8 TB/s HBM peak, algorithmic bytes = every tensor read or written once."""
+    import torch
+
+    import trident_amd
+    from trident_amd import rowops
+
+    y, x = 16384, 8192
+    inp = torch.randn(y, x, device=dev).to(torch.bfloat16).requires_grad_(True)
+    grad = torch.randn(y, x, device=dev).to(torch.bfloat16)
+    mask = (torch.rand(y, x, device=dev) < 0.25).to(torch.uint8)
+    nbytes = y * x * 2
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+
+    def timed(fn, reps=10):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        ev[0].record()
+        for _ in range(reps):
+            fn()
+        ev[1].record()
+        torch.cuda.synchronize()
+        return ev[0].elapsed_time(ev[1]) / reps
+
+    res = {"input": f"bf16 {y} x {x} (256 MiB), softmax along the rows; uint8 mask, 25 % set"}
+    out = trident_amd.function.softmax(inp.detach(), 1)
+    cases = [
+        ("softmax_fwd", lambda: trident_amd.function.softmax(inp.detach(), 1), 2 * nbytes),
+        ("softmax_bwd", lambda: rowops._softmax_backward(grad, out, 1, "kernel.Softmax.backward"), 3 * nbytes),
+        ("masked_softmax_fwd", lambda: trident_amd.function.masked_softmax(inp.detach(), mask, 1), 2 * nbytes + y * x),
+        ("dropout_fwd", lambda: trident_amd.function.dropout(inp.detach(), 0.1), 2 * nbytes),
+    ]
+    for name, fn, moved in cases:
+        ms = timed(fn)
+        gbs = moved / ms / 1e6
+        res[name] = {"ms": round(ms, 4), "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4)}
+    return res
+
+
+def reference_scenario(dev, mode, dtype_name):
+    """The reference's own attention benchmark (benchmarks/benchmark_attention.py:20-57): forward at B=64, H=8, D=64 and
+    backward at B=32, H=8, D=64, sequence lengths 32 ... 512, non-causal, no mask; milliseconds per call for this
+    library, for torch's own GPU attention (the reference's 'torch' backend) and for torch on the host cores."""
+    import torch
+
+    import trident_amd
+
+    dtype = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16}[dtype_name]
+    B = 64 if mode == "forward" else 32
+    H, D = 8, 64
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+
+    def timed(fn, reps=20):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        ev[0].record()
+        for _ in range(reps):
+            fn()
+        ev[1].record()
+        torch.cuda.synchronize()
+        return ev[0].elapsed_time(ev[1]) / reps
+
+    rows = []
+    for S in [2**i for i in range(5, 10)]:
+        g = torch.Generator().manual_seed(S)
+        q, k, v, d_o = [torch.randn(B, H, S, D, generator=g).to(dtype) for _ in range(4)]
+        flops = 4.0 * B * H * S * S * D * (1.0 if mode == "forward" else 2.5)
+        row = {"y_size": S}
+        for backend in ("trident_amd", "torch_gpu", "torch_cpu"):
+            f = trident_amd.function.scaled_dot_product_attention if backend == "trident_amd" else \
+                torch.nn.functional.scaled_dot_product_attention
+            loc = "cpu" if backend == "torch_cpu" else dev
+            tq, tk, tv = [x.to(loc).requires_grad_(mode != "forward") for x in (q, k, v)]
+            tg = d_o.to(loc)
+            if mode == "forward":
+                call = lambda: f(tq, tk, tv)
+            else:
+                out = f(tq, tk, tv)
+                call = lambda: out.backward(tg, retain_graph=True)
+            if backend == "torch_cpu":
+                call()
+                t0 = time.perf_counter()
+                for _ in range(3):
+                    call()
+                ms = (time.perf_counter() - t0) * 1e3 / 3
+            else:
+                ms = timed(call)
+            row[backend + "_ms"] = round(ms, 4)
+            row[backend + "_tflops"] = round(flops / ms / 1e9, 2)
+        rows.append(row)
+    return {"scenario": "attention " + mode, "num_batches": B, "num_heads": H, "x_size": D, "dtype": dtype_name,
+            "cpu_threads": torch.get_num_threads(), "rows": rows,
+            "note": "backward times output.backward(grad, retain_graph=True) as the reference's benchmark does (gradients "
+                    "accumulate into .grad); flops: forward 4 B H S^2 D, backward 10 B H S^2 D"}
+
+
 def ceiling(dev):
     """What the matrix pipe sustains on this box, in this process: MFMA-only loops on random operands (registers;
     A operands from LDS; every LDS read feeding two MFMAs), a large bf16 GEMM, and the three C3 attention kernels."""
@@ -298,6 +398,10 @@ def main():
     ap.add_argument("--workload", default="C3")
     ap.add_argument("--report", action="store_true", help="also print all five configurations on stderr")
     ap.add_argument("--no-configs", action="store_true", help="leave the five-configuration table out of the JSON line")
+    ap.add_argument("--scenario", choices=["attention"], help="instead of the benchmark: the reference's benchmark scenario "
+                    "(benchmarks/benchmarker.py --scenario attention), one JSON line")
+    ap.add_argument("--mode", choices=["forward", "backward"], default="forward")
+    ap.add_argument("--dtype", choices=["float32", "float16", "bfloat16"], default="float16")
     ap.add_argument("--ceiling", action="store_true",
                     help="instead of the benchmark: print one JSON line with the MFMA ceiling of this box (random-operand "
                          "MFMA loops, a bf16 GEMM, the C3 kernels)")
@@ -320,6 +424,9 @@ def main():
     w = workloads.WORKLOADS[a.workload]
     if a.ceiling:
         print(json.dumps({"ceiling": ceiling(dev)}), flush=True)
+        return
+    if a.scenario:
+        print(json.dumps({"reference_scenario": reference_scenario(dev, a.mode, a.dtype)}), flush=True)
         return
     if a.copy_calibration:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
@@ -383,6 +490,7 @@ def main():
         result["cpu_baseline"] = cpu_baseline(w)
     if not a.no_configs:
         result["configs"] = config_figures(dev, not a.no_cpu)
+        result["sibling_ops"] = sibling_ops(dev)
     print(json.dumps(result), flush=True)
 
     if a.report:

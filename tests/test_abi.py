@@ -90,6 +90,29 @@ def test_reference_value_errors():
         trident.util.dtype(torch.int8)
 
 
+def test_reference_limits_can_be_lifted():
+    """config.reference_limits = False: any sequence length and boolean masks get past the argument checks
+    (and then stop at the GPU-only check on this host); head sizes stay powers of two."""
+    f = trident.function.scaled_dot_product_attention
+    y = torch.zeros(2, 4, 12, 16)
+    m = torch.ones(2, 4, 12, 12, dtype=torch.bool)
+    trident.config.reference_limits = False
+    try:
+        with pytest.raises(RuntimeError, match="GPU only"):
+            f(y, y, y)
+        with pytest.raises(RuntimeError, match="GPU only"):
+            f(y, y, y, attn_mask=m)
+        with pytest.raises(ValueError, match="both attn_mask and is_causal"):
+            f(y, y, y, attn_mask=m, is_causal=True)
+        z = torch.zeros(2, 4, 16, 24)
+        with pytest.raises(ValueError, match="power of 2"):
+            f(z, z, z)
+    finally:
+        trident.config.reference_limits = True
+    with pytest.raises(ValueError, match="power of 2"):
+        f(y, y, y)
+
+
 def test_no_cpu_fallback():
     x = torch.zeros(1, 1, 8, 16)
     with pytest.raises(RuntimeError, match="GPU only"):

@@ -311,6 +311,29 @@ def test_dropout_without_causal_or_mask(S, D, device):
     _abi_case(device, torch.bfloat16, S, D, "dropout", 250 + S + D)
 
 
+@pytest.mark.parametrize("dtype,S,D", [(torch.bfloat16, 200, 64), (torch.float32, 100, 32), (torch.float16, 384, 128)])
+def test_operator_without_the_reference_limits(dtype, S, D, device):
+    """config.reference_limits = False: a length that is no power of two and a boolean mask (True = the key takes
+    part, as torch.nn.functional.scaled_dot_product_attention reads it) go through the operator API."""
+    q, k, v, d_o = _gen((2, 2, S, D), 320 + S, dtype)
+    keep = torch.rand(2, 1, S, S, generator=torch.Generator().manual_seed(9)) > 0.3
+    keep[..., 0] = True  # no fully masked row
+    additive = torch.zeros(2, 1, S, S).masked_fill(~keep, float("-inf"))
+    trident.config.reference_limits = False
+    try:
+        _check(device, dtype, q, k, v, d_o, is_causal=True, tag=f"any length S={S}")
+        o, dq, dk, dv, _ = _run(device, q, k, v, d_o, mask=keep)
+    finally:
+        trident.config.reference_limits = True
+    o_ref, _ = parity.oracle_forward(q, k, v, mask=additive)
+    parity.close(o, o_ref, dtype, "bool mask O")
+    dq_r, dk_r, dv_r, _, _ = parity.oracle_backward(q, k, v, d_o, mask=additive, o=o)
+    _, a_dq, a_dk, a_dv = parity.oracle_abs_sums(q, k, v, d_o, mask=additive, o=o)
+    parity.close(dq, dq_r, dtype, "bool mask dQ", a_dq)
+    parity.close(dk, dk_r, dtype, "bool mask dK", a_dk)
+    parity.close(dv, dv_r, dtype, "bool mask dV", a_dv)
+
+
 # ------------------------------------------------------------------ tile counts of the phased kernels
 @pytest.mark.parametrize("variant", ["plain", "causal", "causal+dropout"])
 @pytest.mark.parametrize("S,D", [(256, 128), (768, 128), (1280, 128), (768, 64), (1024, 64)])

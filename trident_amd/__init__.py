@@ -6,6 +6,6 @@ reference's signatures (trident/function/function.py:238-253, trident/operation/
 """
 from . import config, function, operation, util
 from .config import *
-from .module import Attention
+from .module import Attention, Dropout, MaskedSoftmax, Softmax
 
 __version__ = "0.1.0"

@@ -52,6 +52,30 @@ class TriAttnArgs(ctypes.Structure):
     ]
 
 
+class TriRowArgs(ctypes.Structure):
+    """include/tri_rowops.h"""
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("dtype", ctypes.c_int32),
+        ("y_size", ctypes.c_int64),
+        ("x_size", ctypes.c_int64),
+        ("y_stride", ctypes.c_int64),
+        ("x_stride", ctypes.c_int64),
+        ("input", ctypes.c_void_p),
+        ("output", ctypes.c_void_p),
+        ("mask", ctypes.c_void_p),
+        ("mask_dtype", ctypes.c_int32),
+        ("p", ctypes.c_float),
+        ("grad_output", ctypes.c_void_p),
+        ("grad_input", ctypes.c_void_p),
+        ("seed", ctypes.c_uint64),
+        ("offset", ctypes.c_uint64),
+        ("stream", ctypes.c_void_p),
+    ]
+
+
+ROW_EXPORTS = ("tri_softmax_fwd", "tri_softmax_bwd", "tri_dropout_fwd", "tri_dropout_bwd")
+
 EXPORTS = (
     "tri_attn_version",
     "tri_attn_strerror",
@@ -95,6 +119,10 @@ def lib():
             ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
             ctypes.c_void_p, ctypes.c_void_p,
         ]
+        for name in ROW_EXPORTS:
+            fn = getattr(cdll, name)  # AttributeError if a declared symbol is not exported
+            fn.restype = ctypes.c_int
+            fn.argtypes = [ctypes.POINTER(TriRowArgs)]
         cdll.tri_attn_probe_mfma.restype = ctypes.c_int
         cdll.tri_attn_probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
                                              ctypes.c_void_p, ctypes.c_void_p]

@@ -9,7 +9,14 @@ every forward call with dropout (so ``torch.manual_seed`` makes runs repeatable;
 draws a non-deterministic one, trident/operation/attention.py:125). An ``int`` or a
 ``(seed, offset)`` pair fixes the stream: the seed is used as given and the offset advances by
 one per forward call.
+
+``reference_limits``: True keeps the reference's argument rules for attention (sequence length and head size
+powers of two, boolean masks rejected with its error text, trident/operation/attention.py:31-45). False lifts
+the two that the kernels here do not need: any sequence length is accepted, and a boolean mask is taken the way
+torch.nn.functional.scaled_dot_product_attention takes it (True = the key takes part; it becomes an additive
+0 / -inf mask and has no gradient).
 """
 use_autotune = True
 use_trace = False
 dropout_seed = None
+reference_limits = True

@@ -1,9 +1,39 @@
-"""Functional entry points (reference: trident/function/function.py:238-253)."""
+"""Functional entry points (reference: trident/function/function.py:58-67, 166-172, 238-262)."""
 import math
 
 import torch
 
 from . import operation
+
+
+def dropout(input, p=0.5, training=True):
+    """
+    Applies Dropout to an input.
+
+    See Dropout for details.
+    """
+    if training:
+        return operation.Dropout.apply(input.view(-1, input.shape[-1]), p).view(input.shape)
+    else:
+        return input.clone()
+
+
+def masked_softmax(input: torch.Tensor, mask: torch.Tensor, dim: int):
+    """
+    Applies Masked Softmax to an input rescaling them so that an output lie in the range [0,1] and sum to 1.
+
+    See MaskedSoftmax for more details.
+    """
+    return operation.MaskedSoftmax.apply(input, mask, dim)
+
+
+def softmax(input: torch.Tensor, dim: int = None):
+    """
+    Applies Softmax to an input rescaling them so that an output lie in the range [0,1] and sum to 1.
+
+    See Softmax for more details.
+    """
+    return operation.Softmax.apply(input, dim)
 
 
 def scaled_dot_product_attention(

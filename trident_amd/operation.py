@@ -92,12 +92,17 @@ class Attention(torch.autograd.Function):
             raise ValueError("The dimension of query, key and value should be 4.")
 
         if (
-            not util.is_pow2(query.shape[-2])
-            or not util.is_pow2(query.shape[-1])
-            or not util.is_pow2(key.shape[-2])
+            not util.is_pow2(query.shape[-1])
             or not util.is_pow2(key.shape[-1])
-            or not util.is_pow2(value.shape[-2])
             or not util.is_pow2(value.shape[-1])
+            or (
+                config.reference_limits
+                and (
+                    not util.is_pow2(query.shape[-2])
+                    or not util.is_pow2(key.shape[-2])
+                    or not util.is_pow2(value.shape[-2])
+                )
+            )
         ):
             raise ValueError("Attention supports only for power of 2 size tensors.")
 
@@ -105,7 +110,10 @@ class Attention(torch.autograd.Function):
             if is_causal:
                 raise ValueError("Error because both attn_mask and is_causal are set.")
             if mask.dtype == torch.bool:
-                raise ValueError("Boolean mask is not supported yet.")
+                if config.reference_limits:
+                    raise ValueError("Boolean mask is not supported yet.")
+                # torch's meaning of a boolean attn_mask: True = the key takes part in the attention
+                mask = torch.zeros(mask.shape, dtype=query.dtype, device=mask.device).masked_fill_(~mask, float("-inf"))
 
         seed, offset = _next_seed() if dropout_p > 0.0 else (0, 0)
 
@@ -232,3 +240,6 @@ class Attention(torch.autograd.Function):
                 grad_mask = grad_mask.reshape(mask.shape)
 
         return grad_query, grad_key, grad_value, grad_mask
+
+
+from .rowops import Dropout, MaskedSoftmax, Softmax  # noqa: E402,F401  (trident.operation.Softmax etc.)
