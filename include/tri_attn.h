@@ -157,6 +157,12 @@ int tri_attn_bwd(const TriAttnArgs* args);
 #define TRI_ATTN_NOALLOC_MAX_ROWS (1 << 20)
 int tri_attn_bwd_noalloc(const TriAttnArgs* args);
 
+/* Which kernel family a call would run, without launching anything (no counterpart in the reference): pass 0 =
+ * tri_attn_fwd, 1 = tri_attn_bwd_dkdv, 2 = tri_attn_bwd_dq on these arguments. Returns 1 for the matrix-core (MFMA)
+ * kernels (fp16/bf16, D in {64,128}, 16-byte aligned rows; any S without a mask, S a multiple of 128 with one;
+ * no dmask), 0 for the general fp32 vector-ALU kernels, or a negative TRI_ATTN_E* code. */
+int tri_attn_uses_matrix_cores(const TriAttnArgs* args, int pass);
+
 /* Debug / parity helper with no counterpart in the reference (its dropout stream is unpinned):
  * writes the dropout keep decisions (1 = kept) for head index bh, rows [row0,row0+rows),
  * cols [col0,col0+cols) into keep[rows*cols] (device, uint8) using exactly the device code

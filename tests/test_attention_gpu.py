@@ -253,7 +253,23 @@ def test_dropout_extremes_and_determinism(device):
 
 
 # ------------------------------------------------------------------ lengths the operator API rejects
-def _abi_case(device, dtype, S, D, variant, seed, batches=1, heads=2):
+def _assert_kernel_family(q, mask, p, causal, scale, expected):
+    """tri_attn_uses_matrix_cores on the arguments of a call (forward, dK/dV, dQ)."""
+    import ctypes
+    from trident_amd import _lib, operation
+    lse = torch.empty(q.shape[:3], device=q.device, dtype=torch.float32)
+    args = operation._base_args(q, None if mask is None else operation._expand_mask(mask, (*q.shape[:3], q.shape[2])),
+                                p, causal, scale, 0, 0)
+    for name, field in [("q", "q_stride"), ("k", "k_stride"), ("v", "v_stride"), ("o", "o_stride"), ("d_o", "do_stride"),
+                        ("dq", "dq_stride"), ("dk", "dk_stride"), ("dv", "dv_stride")]:
+        operation._fill(args, name, q, field)   # (only pointers' alignment and the strides matter)
+    operation._fill(args, "lse", lse)
+    operation._fill(args, "delta", lse)
+    got = [_lib.lib().tri_attn_uses_matrix_cores(ctypes.byref(args), which) for which in (0, 1, 2)]
+    assert got == [1 if expected else 0] * 3, got
+
+
+def _abi_case(device, dtype, S, D, variant, seed, batches=1, heads=2, matrix_cores=None):
     """The operator API accepts power-of-two lengths only (reference rule); the C ABI takes any
     length.  This calls the ABI wrappers directly: a multiple of 128 that is not one of 256 runs the
     4-wave matrix-core kernels over several tiles, other lengths run the general kernels."""
@@ -274,6 +290,8 @@ def _abi_case(device, dtype, S, D, variant, seed, batches=1, heads=2):
     rng = (977, 3) if p > 0 else (0, 0)
     tq, tk, tv, tdo = [x.to(device) for x in (q, k, v, d_o)]
     tm = None if mask is None else mask.to(device)
+    if matrix_cores is not None:
+        _assert_kernel_family(tq, tm, p, causal, scale, matrix_cores)
     o, lse = Attention._forward(tq, tk, tv, tm, p, causal, scale, *rng)
     delta = torch.full_like(lse, float("nan"))
     dq, dk, dv, _ = Attention._backward(tdo, tq, tk, tv, o, lse, tm, scale, p, causal, *rng, False, delta_out=delta)
@@ -332,6 +350,24 @@ def test_operator_without_the_reference_limits(dtype, S, D, device):
     parity.close(dq, dq_r, dtype, "bool mask dQ", a_dq)
     parity.close(dk, dk_r, dtype, "bool mask dK", a_dk)
     parity.close(dv, dv_r, dtype, "bool mask dV", a_dv)
+
+
+@pytest.mark.parametrize("variant", ["plain", "causal", "dropout", "causal+dropout"])
+@pytest.mark.parametrize("dtype,S,D", [(torch.float16, 32, 64), (torch.bfloat16, 64, 64), (torch.bfloat16, 32, 128),
+                                       (torch.float16, 72, 64), (torch.bfloat16, 200, 128), (torch.bfloat16, 129, 64),
+                                       (torch.float16, 255, 128), (torch.bfloat16, 1000, 64), (torch.bfloat16, 1, 64),
+                                       (torch.float16, 833, 128)])
+def test_any_length_runs_on_the_matrix_cores(dtype, S, D, variant, device):
+    """Lengths that are not multiples of 128 (the reference's benchmark regime S = 32, 64 among them): the 128-row
+    matrix-core kernels with boundary handling (clamped loads, masked keys and rows, guarded stores), not the
+    vector-ALU kernels. Three heads, so that a head's last rows are followed by another head's first ones."""
+    _abi_case(device, dtype, S, D, variant, 600 + S + D, batches=1, heads=3, matrix_cores=True)
+
+
+def test_masked_problems_of_other_lengths_take_the_general_kernels(device):
+    _abi_case(device, torch.bfloat16, 200, 64, "mask", 650, matrix_cores=False)
+    _abi_case(device, torch.float32, 256, 64, "plain", 651, matrix_cores=False)
+    _abi_case(device, torch.bfloat16, 256, 32, "causal", 652, matrix_cores=False)
 
 
 # ------------------------------------------------------------------ tile counts of the phased kernels

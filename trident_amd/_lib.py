@@ -87,6 +87,7 @@ EXPORTS = (
     "tri_attn_bwd",
     "tri_attn_bwd_noalloc",
     "tri_attn_dropout_mask",
+    "tri_attn_uses_matrix_cores",
     "tri_attn_probe_mfma",
 )
 
@@ -113,6 +114,8 @@ def lib():
             fn = getattr(cdll, name)
             fn.restype = ctypes.c_int
             fn.argtypes = [ctypes.POINTER(TriAttnArgs)]
+        cdll.tri_attn_uses_matrix_cores.restype = ctypes.c_int
+        cdll.tri_attn_uses_matrix_cores.argtypes = [ctypes.POINTER(TriAttnArgs), ctypes.c_int]
         cdll.tri_attn_dropout_mask.restype = ctypes.c_int
         cdll.tri_attn_dropout_mask.argtypes = [
             ctypes.c_uint64, ctypes.c_uint64, ctypes.c_float, ctypes.c_uint32,

@@ -37,15 +37,15 @@ FLAGS = [
 
 # The kernels the five benchmark configurations launch (demangled name without the parameter list).
 BASELINE_KERNELS = {
-    "mfma_fwd_kernel<_Float16, 64, 8, false, 0, false>": "C2 fwd",
-    "mfma_fwd_kernel<__bf16, 128, 8, true, 0, false>": "C3 fwd",
+    "mfma_fwd_kernel<_Float16, 64, 8, false, 0, false, false>": "C2 fwd",
+    "mfma_fwd_kernel<__bf16, 128, 8, true, 0, false, false>": "C3 fwd",
     "mfma_dq_phased_kernel<__bf16, 128, true, false, true>": "C3 dQ + delta",
     "mfma_dkdv_phased_kernel<__bf16, 128, true>": "C3 dK/dV",
-    "mfma_fwd_kernel<__bf16, 64, 8, false, 1, false>": "C4 fwd",
+    "mfma_fwd_kernel<__bf16, 64, 8, false, 1, false, false>": "C4 fwd",
     "delta_kernel<__bf16, 64>": "C4 delta",
-    "mfma_dkdv_wide_kernel<__bf16, 64, 8, false, 1, false>": "C4 dK/dV",
-    "mfma_dq_kernel<__bf16, 64, 8, false, 1, false>": "C4 dQ",
-    "mfma_fwd_kernel<__bf16, 128, 8, true, 0, true>": "C5 fwd",
+    "mfma_dkdv_wide_kernel<__bf16, 64, 8, false, 1, false, false>": "C4 dK/dV",
+    "mfma_dq_kernel<__bf16, 64, 8, false, 1, false, false>": "C4 dQ",
+    "mfma_fwd_kernel<__bf16, 128, 8, true, 0, true, false>": "C5 fwd",
     "mfma_dq_phased_kernel<__bf16, 128, true, true, true>": "C5 dQ + delta",
     "mfma_dkdv_pair_kernel<__bf16, 128, true, 0, true>": "C5 dK/dV",
     "generic_fwd_kernel<float, 32>": "C1 fwd",
@@ -125,7 +125,7 @@ def _compile(src):
 
 def resource_table(resources):
     names = _demangle(sorted(resources))
-    rows = sorted((names[m], r) for m, r in resources.items())
+    rows = sorted(((names[m], r) for m, r in resources.items()), key=lambda x: x[0])
     head = f"{'kernel':<64} {'config':<14} {'VGPR':>5} {'AGPR':>5} {'SGPR':>5} {'SGPR spill':>10} {'VGPR spill':>10} " \
            f"{'scratch B':>9} {'LDS B':>7} {'waves/SIMD':>10}"
     out = [head]

@@ -242,6 +242,14 @@ int tri_attn_bwd_noalloc(const TriAttnArgs* args) {
     return tri_attn_bwd(&a);
 }
 
+int tri_attn_uses_matrix_cores(const TriAttnArgs* args, int pass) {
+    if (pass < 0 || pass > 2) return TRI_ATTN_ESHAPE;
+    KParams p;
+    const int rc = make_params(args, pass == 0 ? 1 : (pass == 1 ? 4 : 8), &p);
+    if (rc) return rc;
+    return mfma_supported(pass == 0 ? kMfmaFwd : (pass == 1 ? kMfmaDkdv : kMfmaDq), args->dtype, p) ? 1 : 0;
+}
+
 int tri_attn_dropout_mask(uint64_t seed, uint64_t offset, float dropout_p, uint32_t bh, int32_t row0, int32_t rows,
                           int32_t col0, int32_t cols, uint8_t* keep, void* stream) {
     if (keep == nullptr) return TRI_ATTN_ENULL;

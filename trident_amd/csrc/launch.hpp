@@ -11,7 +11,7 @@ enum GenericKernel { kGenericFwd = 0, kGenericDelta = 1, kGenericDkdv = 2, kGene
 // generic.hip: any shape / dtype, vector-ALU fp32 arithmetic.
 int launch_generic_any(int which, int dtype, const KParams& p, hipStream_t stream);
 
-// mfma_*.hip: fp16/bf16, D in {64,128}, S a multiple of 128, 16-byte aligned rows.
+// mfma_*.hip: fp16/bf16, D in {64,128}, 16-byte aligned rows; any S without a mask, S a multiple of 128 with one.
 enum MfmaKernel { kMfmaFwd = 0, kMfmaDkdv = 1, kMfmaDq = 2 };
 bool mfma_supported(int which, int dtype, const KParams& p);
 int launch_mfma_fwd(int dtype, const KParams& p, hipStream_t stream);

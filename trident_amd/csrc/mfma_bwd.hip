@@ -36,8 +36,11 @@ __device__ __forceinline__ float mask_at(const void* mask, int64_t off) {
 // staging registers, no ds_write). Per 32-key block: S^T = K Q^T and dP^T = V dO^T from row
 // fragments, dS^T = P^T (dP^T - delta) on the vector ALU, dQ^T += K^T dS^T with K^T read through
 // transposed LDS reads of the same K tile.
-template <typename T, int D, int NW, bool CAUSAL, int MASK, bool DROPOUT>
+// RAGGED (4 waves, no mask): S is not a multiple of 128. Rows and keys at or beyond S do not exist: loads clamp
+// their row index to S - 1, keys >= S get probability 0, rows >= S are not stored.
+template <typename T, int D, int NW, bool CAUSAL, int MASK, bool DROPOUT, bool RAGGED = false>
 __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
+    static_assert(!RAGGED || (NW == 4 && MASK == 0), "ragged lengths: 4 waves, no mask");
     using Tile = SwzTile<D>;
     constexpr int kRows = 32 * NW;
     constexpr int kStages = 4;
@@ -59,14 +62,15 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63, l32 = lane & 31, h = lane >> 5;
     int bh, qt;
-    map_block_for<MASK>(p, blockIdx.x, p.S / kRows, CAUSAL ? kHeavyLast : kUniformTiles, &bh, &qt);
+    map_block_for<MASK>(p, blockIdx.x, (p.S + kRows - 1) / kRows, CAUSAL ? kHeavyLast : kUniformTiles, &bh, &qt);
     const int b = bh / p.H, hd = bh % p.H;
     const int q0 = qt * kRows;
     const int wrow0 = q0 + 32 * wave;
     const int qrow = wrow0 + l32;
+    const int qrow_ld = RAGGED ? min(qrow, p.S - 1) : qrow;  // (a row that does not exist reads the last one)
 
-    const char* qrowp = static_cast<const char*>(p.q) + (b * p.qs[0] + hd * p.qs[1] + static_cast<int64_t>(qrow) * p.qs[2]) * 2;
-    const char* gorowp = static_cast<const char*>(p.d_o) + (b * p.dos[0] + hd * p.dos[1] + static_cast<int64_t>(qrow) * p.dos[2]) * 2;
+    const char* qrowp = static_cast<const char*>(p.q) + (b * p.qs[0] + hd * p.qs[1] + static_cast<int64_t>(qrow_ld) * p.qs[2]) * 2;
+    const char* gorowp = static_cast<const char*>(p.d_o) + (b * p.dos[0] + hd * p.dos[1] + static_cast<int64_t>(qrow_ld) * p.dos[2]) * 2;
     const char* kbase = static_cast<const char*>(p.k) + (b * p.ks[0] + hd * p.ks[1]) * 2;
     const char* vbase = static_cast<const char*>(p.v) + (b * p.vs[0] + hd * p.vs[1]) * 2;
     const int64_t krow_bytes = p.ks[2] * 2, vrow_bytes = p.vs[2] * 2;
@@ -77,16 +81,17 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
         qf[kk] = *reinterpret_cast<const u32x4*>(qrowp + (2 * kk + h) * 16);
         gf[kk] = *reinterpret_cast<const u32x4*>(gorowp + (2 * kk + h) * 16);
     }
-    float lse = p.lse[static_cast<int64_t>(bh) * p.S + qrow];
-    const float dlt = p.delta[static_cast<int64_t>(bh) * p.S + qrow];
+    float lse = p.lse[static_cast<int64_t>(bh) * p.S + qrow_ld];
+    const float dlt = p.delta[static_cast<int64_t>(bh) * p.S + qrow_ld];
     const float c = p.scale_log2;
 
     f32x16 acc[DB];
 #pragma unroll
     for (int db = 0; db < DB; ++db) acc[db] = zero16();
 
-    const int n_tiles = CAUSAL ? (q0 + kRows) / kBN : p.S / kBN;        // tiles the workgroup streams
-    const int my_tiles = CAUSAL ? (wrow0 + 31) / kBN + 1 : n_tiles;     // tiles with keys visible to this wave
+    const int num_key_tiles = (p.S + kBN - 1) / kBN;
+    const int n_tiles = CAUSAL ? min((q0 + kRows) / kBN, num_key_tiles) : num_key_tiles;  // tiles the workgroup streams
+    const int my_tiles = CAUSAL ? min((wrow0 + 31) / kBN + 1, n_tiles) : n_tiles;         // tiles with keys visible to this wave
 
     int src_off[kBlocksPerWave];
 #pragma unroll
@@ -103,7 +108,11 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
             const bool is_v = blk >= Tile::kBlocks;
             const char* tile_src = is_v ? vbase + static_cast<int64_t>(t) * kBN * vrow_bytes
                                         : kbase + static_cast<int64_t>(t) * kBN * krow_bytes;
-            lds_direct_load16(tile_src, src_off[i], stage + blk * 1024);
+            if (RAGGED && (t + 1) * kBN > p.S)  // the sequence ends inside this tile
+                lds_direct_load16(tile_src, Tile::src_off_clamped(is_v ? blk - Tile::kBlocks : blk, lane, is_v ? vrow_bytes : krow_bytes,
+                                                                  p.S - 1 - t * kBN), stage + blk * 1024);
+            else
+                lds_direct_load16(tile_src, src_off[i], stage + blk * 1024);
         }
     };
     char* mask_lds = smem + kStages * kStageBytes + wave * kMaskBytes;
@@ -200,6 +209,10 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) st[i] = t0 + 32 * kb + c_row(i, h) <= qrow ? st[i] : -INFINITY;
             }
+            if (RAGGED && !CAUSAL && t0 + 32 * kb + 32 > p.S) {  // keys that do not exist
+#pragma unroll
+                for (int i = 0; i < 16; ++i) st[i] = t0 + 32 * kb + c_row(i, h) < p.S ? st[i] : -INFINITY;
+            }
             float ds[16];
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
@@ -238,7 +251,8 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
         static_assert(NW * Store::kPatchBytes <= kStages * kStageBytes, "patches must fit into the ring");
         char* out0 = static_cast<char*>(p.dq) + (b * p.dqs[0] + hd * p.dqs[1] + static_cast<int64_t>(wrow0) * p.dqs[2]) * 2;
         const float sc = p.scale;
-        Store::run(acc, [sc](float x) { return x * sc; }, smem + wave * Store::kPatchBytes, out0, p.dqs[2] * 2, lane);
+        Store::run(acc, [sc](float x) { return x * sc; }, smem + wave * Store::kPatchBytes, out0, p.dqs[2] * 2, lane,
+                   RAGGED ? p.S - wrow0 : 32);
     }
 }
 
@@ -517,8 +531,12 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
 // tiles (plus their lse and delta) in a ring of 4 filled by LDS-direct loads three tiles ahead.
 // Per 32-row query block: S = Q K^T and dP = dO V^T from row fragments, P and dS on the vector
 // ALU, dV^T += dO^T P and dK^T += Q^T dS with the transposed LDS reads of the same tiles.
-template <typename T, int D, int NW, bool CAUSAL, int MASK, bool DROPOUT>
-__global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParams p) {
+// RAGGED (4 waves, no mask; also serves D = 128, one workgroup per CU): S is not a multiple of 128. Loads clamp their
+// row index to S - 1, query rows >= S get probability 0 (they would otherwise add the last row once more), keys >= S
+// are not stored.
+template <typename T, int D, int NW, bool CAUSAL, int MASK, bool DROPOUT, bool RAGGED = false>
+__global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel(const KParams p) {
+    static_assert(!RAGGED || (NW == 4 && MASK == 0), "ragged lengths: 4 waves, no mask");
     using Tile = SwzTile<D>;
     constexpr int kKeys = 32 * NW;
     constexpr int kStages = 4;
@@ -541,11 +559,12 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63, l32 = lane & 31, h = lane >> 5;
     int bh, kt;
-    map_block_for<MASK>(p, blockIdx.x, p.S / kKeys, CAUSAL ? kHeavyFirst : kUniformTiles, &bh, &kt);
+    map_block_for<MASK>(p, blockIdx.x, (p.S + kKeys - 1) / kKeys, CAUSAL ? kHeavyFirst : kUniformTiles, &bh, &kt);
     const int b = bh / p.H, hd = bh % p.H;
     const int k0 = kt * kKeys;
     const int wkey0 = k0 + 32 * wave;
     const int key = wkey0 + l32;
+    const int key_ld = RAGGED ? min(key, p.S - 1) : key;  // (a key that does not exist reads the last one)
 
     const char* kbase = static_cast<const char*>(p.k) + (b * p.ks[0] + hd * p.ks[1]) * 2;
     const char* vbase = static_cast<const char*>(p.v) + (b * p.vs[0] + hd * p.vs[1]) * 2;
@@ -558,8 +577,8 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
     u32x4 kf[KK], vf[KK];
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
-        kf[kk] = *reinterpret_cast<const u32x4*>(kbase + static_cast<int64_t>(key) * p.ks[2] * 2 + (2 * kk + h) * 16);
-        vf[kk] = *reinterpret_cast<const u32x4*>(vbase + static_cast<int64_t>(key) * p.vs[2] * 2 + (2 * kk + h) * 16);
+        kf[kk] = *reinterpret_cast<const u32x4*>(kbase + static_cast<int64_t>(key_ld) * p.ks[2] * 2 + (2 * kk + h) * 16);
+        vf[kk] = *reinterpret_cast<const u32x4*>(vbase + static_cast<int64_t>(key_ld) * p.vs[2] * 2 + (2 * kk + h) * 16);
     }
     const float c = p.scale_log2;
 
@@ -579,9 +598,11 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
     }
     const int t_begin = CAUSAL ? k0 / kBN : 0;                  // first tile with rows that see the workgroup's keys
     const int my_begin = CAUSAL ? wkey0 / kBN : 0;              // first tile with rows that see this wave's keys
-    const int n_tiles = p.S / kBN;
+    const int n_tiles = (p.S + kBN - 1) / kBN;
     auto issue_tile = [&](int t) {
         char* stage = smem + (t % kStages) * kStageBytes;
+        const bool partial = RAGGED && (t + 1) * kBN > p.S;  // the sequence ends inside this tile
+        const int last = p.S - 1 - t * kBN;
 #pragma unroll
         for (int i = 0; i < kBlocksPerWave; ++i) {
             const int blk = wave * kBlocksPerWave + i;
@@ -589,13 +610,17 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
             const char* tile_src = is_g ? gbase + static_cast<int64_t>(t) * kBN * grow_bytes
                                         : qbase + static_cast<int64_t>(t) * kBN * qrow_bytes;
             char* dst = stage + (is_g ? Tile::kBytes + (blk - Tile::kBlocks) * 1024 : blk * 1024);
-            lds_direct_load16(tile_src, src_off[i], dst);
+            if (partial)
+                lds_direct_load16(tile_src, Tile::src_off_clamped(is_g ? blk - Tile::kBlocks : blk, lane, is_g ? grow_bytes : qrow_bytes, last), dst);
+            else
+                lds_direct_load16(tile_src, src_off[i], dst);
         }
         // every wave issues exactly one more load, so that the vmcnt bookkeeping is the same in all of
         // them: even waves fetch the 64 lse values, odd waves the 64 delta values (duplicates land
         // on the same bytes)
-        if (wave & 1) lds_direct_load4(delta_base + t * kBN, lane * 4, stage + 2 * Tile::kBytes + kBN * 4);
-        else lds_direct_load4(lse_base + t * kBN, lane * 4, stage + 2 * Tile::kBytes);
+        const int aux = (partial ? min(lane, last) : lane) * 4;
+        if (wave & 1) lds_direct_load4(delta_base + t * kBN, aux, stage + 2 * Tile::kBytes + kBN * 4);
+        else lds_direct_load4(lse_base + t * kBN, aux, stage + 2 * Tile::kBytes);
     };
     char* mask_lds = smem + kStages * kStageBytes + wave * MaskTile::kBytes;
     auto issue_mask = [&](int t) {  // rows of tile t x this wave's keys -> the wave's region
@@ -686,6 +711,10 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
 #pragma unroll
                 for (int i = 0; i < 16; ++i) s[i] = key <= rb + c_row(i, h) ? s[i] : -INFINITY;
             }
+            if (RAGGED && rb + 32 > p.S) {  // query rows that do not exist contribute nothing
+#pragma unroll
+                for (int i = 0; i < 16; ++i) s[i] = rb + c_row(i, h) < p.S ? s[i] : -INFINITY;
+            }
             u32x4 pb[2], sb[2];
             {
                 float pr[16], ds[16];
@@ -752,9 +781,10 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dkdv_wide_kernel(const KParam
         char* dk0 = static_cast<char*>(p.dk) + (b * p.dks[0] + hd * p.dks[1] + static_cast<int64_t>(wkey0) * p.dks[2]) * 2;
         char* dv0 = static_cast<char*>(p.dv) + (b * p.dvs[0] + hd * p.dvs[1] + static_cast<int64_t>(wkey0) * p.dvs[2]) * 2;
         const float sc = p.scale;
-        Store::run(dk, [sc](float x) { return x * sc; }, patch, dk0, p.dks[2] * 2, lane);
+        const int keys_here = RAGGED ? p.S - wkey0 : 32;
+        Store::run(dk, [sc](float x) { return x * sc; }, patch, dk0, p.dks[2] * 2, lane, keys_here);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // patch read before it is rewritten
-        Store::run(dv, [](float x) { return x; }, patch, dv0, p.dvs[2] * 2, lane);
+        Store::run(dv, [](float x) { return x; }, patch, dv0, p.dvs[2] * 2, lane, keys_here);
     }
 }
 
@@ -1506,7 +1536,14 @@ int launch_dq_dropout(const KParams& p, hipStream_t stream, bool with_delta) {
     if (with_delta) return TRI_ATTN_ESHAPE;  // (callers ask dq_fuses_delta first)
     // 8 waves (256 query rows) when the sequence allows it, else 4 waves (128 rows)
     if (p.S % 256 == 0) return launch_dq_waves<T, D, 8, CAUSAL, MASK>(p, stream);
-    return launch_dq_waves<T, D, 4, CAUSAL, MASK>(p, stream);
+    if (p.S % 128 == 0) return launch_dq_waves<T, D, 4, CAUSAL, MASK>(p, stream);
+    if constexpr (MASK == kNoMask) {  // any other length: 128-row workgroups with boundary handling
+        const dim3 grid(p.B * p.H * ((p.S + 127) / 128)), block(256);
+        if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dq_kernel<T, D, 4, CAUSAL, kNoMask, true, true>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((mfma_dq_kernel<T, D, 4, CAUSAL, kNoMask, false, true>), grid, block, 0, stream, p);
+        return static_cast<int>(hipGetLastError());
+    }
+    return TRI_ATTN_ESHAPE;  // (mfma_supported keeps masked problems of such lengths away)
 }
 
 template <typename T, int D, int NW, bool CAUSAL, int MASK>
@@ -1519,6 +1556,17 @@ int launch_dkdv_waves(const KParams& p, hipStream_t stream) {
 
 template <typename T, int D, bool CAUSAL, int MASK>
 int launch_dkdv_dropout(const KParams& p, hipStream_t stream) {
+    if (p.S % 128 != 0) {
+        // any length (no mask): 128-key workgroups of the 32-keys-per-wave kernel with boundary handling, for both
+        // head sizes (at D = 128 with the whole register file, one workgroup per CU)
+        if constexpr (MASK == kNoMask) {
+            const dim3 grid(p.B * p.H * ((p.S + 127) / 128)), block(256);
+            if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dkdv_wide_kernel<T, D, 4, CAUSAL, kNoMask, true, true>), grid, block, 0, stream, p);
+            else hipLaunchKernelGGL((mfma_dkdv_wide_kernel<T, D, 4, CAUSAL, kNoMask, false, true>), grid, block, 0, stream, p);
+            return static_cast<int>(hipGetLastError());
+        }
+        return TRI_ATTN_ESHAPE;  // (mfma_supported keeps masked problems of such lengths away)
+    }
     if constexpr (D == 64) {
         // the two-waves-per-SIMD kernel fits its registers: 8 waves (256 keys) when the sequence
         // allows it, else 4 waves (128 keys)

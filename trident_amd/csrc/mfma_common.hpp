@@ -179,6 +179,14 @@ struct SwzTile {
         const int c = (lane % kChunks) ^ swz(row);
         return row * row_stride_bytes + c * 16;
     }
+    // The same for a tile whose rows beyond `last_row` (tile-relative, >= 0) do not exist (the sequence ends inside
+    // the tile): such lanes fetch the last existing row instead, same chunk, so nothing outside the tensor is read
+    // and the tile holds harmless copies that the kernels mask out.
+    static __device__ __forceinline__ uint32_t src_off_clamped(int blk, int lane, int64_t row_stride_bytes, int last_row) {
+        const int row = blk * kRowsPerBlock + lane / kChunks;
+        const int c = (lane % kChunks) ^ swz(row);
+        return static_cast<uint32_t>((row < last_row ? row : last_row) * row_stride_bytes + c * 16);
+    }
     // byte offset (within the tile) a lane passes to the transposed read of column block db
     // (32 columns), half = 0/1 (K-slots 0-3 / 4-7); add ks * 16 * kRowBytes for K-step ks
     static __device__ __forceinline__ int tr_off(int db, int half, int lane) {
@@ -292,9 +300,10 @@ struct RowBlockStore {
     static constexpr int kPatchBytes = 32 * kPitch;
     static constexpr int kLanesPerRow = kRowBytes / 16;
     static constexpr int kRowsPerStore = 64 / kLanesPerRow;
+    // `rows`: how many of the wave's 32 rows exist (the others are not stored).
     template <typename Scale>
     static __device__ __forceinline__ void run(const f32x16 (&acc)[NB], Scale scale, char* patch, char* row0,
-                                               int64_t row_stride_bytes, int lane) {
+                                               int64_t row_stride_bytes, int lane, int rows = 32) {
         const int l32 = lane & 31, h = lane >> 5;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
@@ -311,7 +320,7 @@ struct RowBlockStore {
         for (int i = 0; i < 32 / kRowsPerStore; ++i) {
             const int row = i * kRowsPerStore + r;
             const u32x4 v = lds_read16(patch, row * kPitch + c * 16);
-            *reinterpret_cast<u32x4*>(row0 + row * row_stride_bytes + c * 16) = v;
+            if (row < rows) *reinterpret_cast<u32x4*>(row0 + row * row_stride_bytes + c * 16) = v;
         }
     }
 };

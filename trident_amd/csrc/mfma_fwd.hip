@@ -1,5 +1,5 @@
 // Forward attention on the matrix cores: online-softmax flash kernel for fp16/bf16,
-// D in {64,128}, S a multiple of 128 (replaces trident/kernel/attention.py:33-165).
+// D in {64,128}; any S without a mask, multiples of 128 with one (replaces trident/kernel/attention.py:33-165).
 //
 // A workgroup of NW waves owns 32*NW query rows, one wave 32 of them. Q stays in registers as
 // the B operand of S^T = K Q^T; K and V tiles of 64 keys live row-major (swizzled) in a four-stage
@@ -33,8 +33,11 @@ constexpr float kTau = 8.f;  // lazy-rescale threshold, log2 domain
 
 enum MaskKind { kNoMask = 0, kMaskF32 = 1, kMaskT = 2 };
 
-template <typename T, int D, int NW, bool CAUSAL, int MASK, bool DROPOUT>
+// RAGGED (4 waves, no mask): S is not a multiple of 128. Query rows and keys at or beyond S do not exist: row and
+// tile loads clamp their row index to S - 1, the scores of keys >= S are set to -inf, and rows >= S are not stored.
+template <typename T, int D, int NW, bool CAUSAL, int MASK, bool DROPOUT, bool RAGGED = false>
 __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
+    static_assert(!RAGGED || (NW == 4 && MASK == 0), "ragged lengths: 4 waves, no mask");
     using Tile = SwzTile<D>;
     constexpr int kBM = 32 * NW;
     constexpr int kKBytes = Tile::kBytes;
@@ -71,8 +74,10 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     constexpr int kOrder = CAUSAL ? kHeavyLast : kUniformTiles;
     int round = 0;
     int bh, qt;
-    if constexpr (kPersistent) map_item(blockIdx.x, gridDim.x, 0, p.B * p.H, p.S / kBM, kOrder, &bh, &qt);
-    else map_block_for<MASK>(p, blockIdx.x, p.S / kBM, kOrder, &bh, &qt);
+    const int num_row_tiles = (p.S + kBM - 1) / kBM;
+    const int num_key_tiles = (p.S + kBN - 1) / kBN;
+    if constexpr (kPersistent) map_item(blockIdx.x, gridDim.x, 0, p.B * p.H, num_row_tiles, kOrder, &bh, &qt);
+    else map_block_for<MASK>(p, blockIdx.x, num_row_tiles, kOrder, &bh, &qt);
     int b, hd, wrow0, qrow, n_tiles, my_tiles;
     const char *kbase, *vbase;
     const int64_t krow_bytes = p.ks[2] * 2, vrow_bytes = p.vs[2] * 2;
@@ -83,14 +88,15 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
         const int q0 = qt * kBM;
         wrow0 = q0 + 32 * wave;  // first query row of this wave
         qrow = wrow0 + l32;
+        const int qrow_ld = RAGGED ? min(qrow, p.S - 1) : qrow;  // (a row that does not exist reads the last one)
         const char* qbase = static_cast<const char*>(p.q) + (b * p.qs[0] + hd * p.qs[1]) * 2;
         kbase = static_cast<const char*>(p.k) + (b * p.ks[0] + hd * p.ks[1]) * 2;
         vbase = static_cast<const char*>(p.v) + (b * p.vs[0] + hd * p.vs[1]) * 2;
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk)
-            qf[kk] = *reinterpret_cast<const u32x4*>(qbase + qrow * p.qs[2] * 2 + (2 * kk + h) * 16);
-        n_tiles = CAUSAL ? (q0 + kBM) / kBN : p.S / kBN;       // tiles the workgroup streams
-        my_tiles = CAUSAL ? (wrow0 + 31) / kBN + 1 : n_tiles;  // tiles this wave has visible keys in
+            qf[kk] = *reinterpret_cast<const u32x4*>(qbase + qrow_ld * p.qs[2] * 2 + (2 * kk + h) * 16);
+        n_tiles = CAUSAL ? min((q0 + kBM) / kBN, num_key_tiles) : num_key_tiles;  // tiles the workgroup streams
+        my_tiles = CAUSAL ? min((wrow0 + 31) / kBN + 1, n_tiles) : n_tiles;       // tiles this wave has visible keys in
     };
     set_item();
 
@@ -124,7 +130,15 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     auto issue_load = [&](int t, int idx) {
         char* stage = smem + (t % kStages) * kStageBytes + wave * 1024;
         const int i = idx % kPerOperand;
-        if (idx < kPerOperand)
+        if (RAGGED && (t + 1) * kBN > p.S) {  // the sequence ends inside this tile: clamped rows, offsets from the tile's first row
+            const int last = p.S - 1 - t * kBN;
+            if (idx < kPerOperand)
+                lds_direct_load16(kbase + static_cast<int64_t>(t) * kBN * krow_bytes,
+                                  Tile::src_off_clamped(wave + i * NW, lane, krow_bytes, last), stage + i * NW * 1024);
+            else
+                lds_direct_load16(vbase + static_cast<int64_t>(t) * kBN * vrow_bytes,
+                                  Tile::src_off_clamped(wave + i * NW, lane, vrow_bytes, last), stage + kKBytes + i * NW * 1024);
+        } else if (idx < kPerOperand)
             lds_direct_load16(kbase + (static_cast<int64_t>(t) * kBN + i * kRowStep) * krow_bytes, koff, stage + i * NW * 1024);
         else
             lds_direct_load16(vbase + (static_cast<int64_t>(t) * kBN + i * kRowStep) * vrow_bytes, voff, stage + kKBytes + i * NW * 1024);
@@ -340,6 +354,13 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
                     x[e] = key <= qrow ? x[e] : -INFINITY;
                 }
             }
+            if (RAGGED && !CAUSAL && t0 + kBN > p.S) {  // keys that do not exist (under the causal mask no existing row sees them)
+#pragma unroll
+                for (int e = 0; e < 32; ++e) {
+                    const int key = t0 + 32 * (e >> 4) + c_row(e & 15, h);
+                    x[e] = key < p.S ? x[e] : -INFINITY;
+                }
+            }
             float mx = x[0], mx1 = x[16];  // two chains: a dependent maximum waits out the ALU latency
 #pragma unroll
             for (int e = 1; e < 16; ++e) {
@@ -482,12 +503,21 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
         for (int cb = 0; cb < DB / 2; ++cb) {
             if (cb) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // patch read before it is rewritten
             const f32x16(&part)[2] = *reinterpret_cast<const f32x16(*)[2]>(&oacc[2 * cb]);
-            Store::run(part, [inv](float x) { return x * inv; }, patch, o0 + cb * 128, p.os[2] * 2, lane);
+            Store::run(part, [inv](float x) { return x * inv; }, patch, o0 + cb * 128, p.os[2] * 2, lane,
+                       RAGGED ? p.S - wrow0 : 32);
         }
     }
-    if (h == 0) *lse_out = m + fast_log2(l);
+    if (h == 0 && (!RAGGED || qrow < p.S)) *lse_out = m + fast_log2(l);
     if (!more) break;
     }
+}
+
+template <typename T, int D, bool CAUSAL>
+int launch_fwd_ragged(const KParams& p, hipStream_t stream) {
+    const dim3 grid(p.B * p.H * ((p.S + 127) / 128)), block(256);
+    if (p.thr8 > 0) hipLaunchKernelGGL((mfma_fwd_kernel<T, D, 4, CAUSAL, kNoMask, true, true>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((mfma_fwd_kernel<T, D, 4, CAUSAL, kNoMask, false, true>), grid, block, 0, stream, p);
+    return static_cast<int>(hipGetLastError());
 }
 
 template <typename T, int D, int NW, bool CAUSAL, int MASK>
@@ -513,7 +543,9 @@ template <typename T, int D>
 int launch_fwd_waves(int dtype, const KParams& p, hipStream_t stream) {
     // 8 waves (256 query rows) when the sequence allows it: two waves per SIMD out of phase
     if (p.S % 256 == 0) return launch_fwd_variant<T, D, 8>(dtype, p, stream);
-    return launch_fwd_variant<T, D, 4>(dtype, p, stream);
+    if (p.S % 128 == 0) return launch_fwd_variant<T, D, 4>(dtype, p, stream);
+    // any other length (no mask: mfma_supported): 128-row workgroups with boundary handling
+    return p.causal ? launch_fwd_ragged<T, D, true>(p, stream) : launch_fwd_ragged<T, D, false>(p, stream);
 }
 
 }  // namespace

@@ -53,7 +53,8 @@ static bool tile_offsets_fit(const int64_t* strides) { return strides[2] >= 0 &&
 bool mfma_supported(int which, int dtype, const KParams& p) {
     if (dtype != TRI_ATTN_F16 && dtype != TRI_ATTN_BF16) return false;
     if (p.D != 64 && p.D != 128) return false;
-    if (p.S % 128 != 0) return false;
+    // lengths that are not multiples of 128 run the 4-wave kernels with boundary handling; those read no mask
+    if (p.S % 128 != 0 && (p.mask != nullptr || p.dmask != nullptr)) return false;
     if (!(p.scale > 0.f)) return false;  // the kernels take row maxima before scaling
     if (!aligned16(p.q) || !aligned16(p.k) || !aligned16(p.v)) return false;
     if (!strides8(p.qs) || !strides8(p.ks) || !strides8(p.vs)) return false;
