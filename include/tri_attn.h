@@ -90,7 +90,9 @@ typedef struct TriAttnArgs {
     void* dq;                  /* grad_query_ptr (need not be zeroed) */
     void* dk;                  /* grad_key_ptr */
     void* dv;                  /* grad_value_ptr */
-    void* dmask;               /* grad_mask_ptr or NULL: dense [B,H,S,S] in mask_dtype, dS per head */
+    void* dmask;               /* grad_mask_ptr or NULL: logical [B,H,S,S] through dmask_stride, in mask_dtype. A stride of 0
+                                  sums the gradient over that dimension (a broadcast mask): the buffer must then be fp32 and
+                                  zero-filled by the caller, and the kernels add to it atomically (order of summation not fixed) */
     float* delta;              /* delta_ptr, fp32 [B,H,S]: written by bwd_delta, read by dkdv/dq */
 
     int64_t q_stride[4];
@@ -159,8 +161,8 @@ int tri_attn_bwd_noalloc(const TriAttnArgs* args);
 
 /* Which kernel family a call would run, without launching anything (no counterpart in the reference): pass 0 =
  * tri_attn_fwd, 1 = tri_attn_bwd_dkdv, 2 = tri_attn_bwd_dq on these arguments. Returns 1 for the matrix-core (MFMA)
- * kernels (fp16/bf16, D in {64,128}, 16-byte aligned rows; any S without a mask, S a multiple of 128 with one;
- * no dmask), 0 for the general fp32 vector-ALU kernels, or a negative TRI_ATTN_E* code. */
+ * kernels (fp16/bf16, D in {64,128}, 16-byte aligned rows; any S without a mask, S a multiple of 128
+ * with one), 0 for the general fp32 vector-ALU kernels, or a negative TRI_ATTN_E* code. */
 int tri_attn_uses_matrix_cores(const TriAttnArgs* args, int pass);
 
 /* Debug / parity helper with no counterpart in the reference (its dropout stream is unpinned):

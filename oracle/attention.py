@@ -132,7 +132,7 @@ def attention_backward(q, k, v, d_out, mask=None, dropout_p=0.0, is_causal=False
             if dmask is not None:
                 mb = 0 if mask.shape[0] == 1 else b
                 mh = 0 if mask.shape[1] == 1 else h
-                dmask[mb, mh] += ds
+                dmask[mb, mh] += ds.sum(axis=0, keepdims=True) if mask.shape[2] == 1 else ds  # (row-broadcast mask)
     return dq, dk, dv, dmask, delta
 
 

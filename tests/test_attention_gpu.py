@@ -172,6 +172,36 @@ def test_key_padding_mask_row_broadcast(dtype, device):
     _check(device, dtype, q, k, v, d_o, mask=mask, tag="key-padding")
 
 
+@pytest.mark.parametrize("dtype,mask_dtype,mshape", [(torch.bfloat16, torch.bfloat16, (2, 3, 256, 256)),
+                                                     (torch.bfloat16, torch.float32, (2, 1, 256, 256)),
+                                                     (torch.float16, torch.float16, (1, 3, 256, 256)),
+                                                     (torch.bfloat16, torch.float32, (2, 1, 1, 256)),
+                                                     (torch.float32, torch.float32, (1, 1, 1, 256))])
+@pytest.mark.parametrize("D", [64, 128])
+def test_mask_gradient_on_the_matrix_cores(dtype, mask_dtype, mshape, D, device):
+    """The mask gradient from the matrix-core dQ kernel (16-bit problems): written in place for a full mask, added
+    atomically into the mask's own shape for masks broadcast over batch, heads or rows (a key-padding mask with a
+    gradient among them), in the mask's dtype. The fp32 problem runs the general kernels on the same contract."""
+    import ctypes
+    from trident_amd import _lib, operation
+    B, H, S = 2, 3, 256
+    q, k, v, d_o = _gen((B, H, S, D), 37 + D, dtype)
+    mask = (0.5 * torch.randn(*mshape, generator=torch.Generator().manual_seed(38))).to(mask_dtype)
+    _check(device, dtype, q, k, v, d_o, mask=mask, mask_grad=True, tag=f"dmask {mshape} {mask_dtype}")
+    # which kernel family writes it
+    tq = q.to(device)
+    buf = torch.zeros(mshape, device=device, dtype=torch.float32 if mshape != (B, H, S, S) else mask_dtype)
+    mview = operation._expand_mask(mask.to(device).to(buf.dtype), (B, H, S, S))
+    args = operation._base_args(tq, mview, 0.0, False, 0.125, 0, 0)
+    for name, field in [("q", "q_stride"), ("k", "k_stride"), ("v", "v_stride"), ("d_o", "do_stride"), ("dq", "dq_stride")]:
+        operation._fill(args, name, tq, field)
+    lse = torch.empty(B, H, S, device=device)
+    operation._fill(args, "lse", lse)
+    operation._fill(args, "delta", lse)
+    operation._fill(args, "dmask", buf.expand(B, H, S, S), "dmask_stride")
+    assert _lib.lib().tri_attn_uses_matrix_cores(ctypes.byref(args), 2) == (0 if dtype == torch.float32 else 1)
+
+
 @pytest.mark.parametrize("D", [64, 128])
 def test_fp32_mask_many_tiles(D, device):
     """fp32 mask shared by the heads over 8 key tiles and 2 workgroups per head: the staged mask path (D=64)

@@ -124,10 +124,11 @@ def test_against_torch_sdpa_reference_shapes(shape, causal):
         np.testing.assert_allclose(a, b, rtol=0, atol=1e-10)
 
 
-def test_broadcast_mask_gradient_matches_autograd():
+@pytest.mark.parametrize("mshape", [(3, 1, 16, 16), (1, 4, 16, 16), (3, 1, 1, 16), (1, 1, 1, 16)])
+def test_broadcast_mask_gradient_matches_autograd(mshape):
     shape = (3, 4, 16, 8)
     q, k, v, d_o = [_rand(shape, s) for s in (1, 2, 3, 4)]
-    mask = _rand((3, 1, 16, 16), 5)
+    mask = _rand(mshape, 5)
     _, _, _, _, dm_t = _torch_sdpa(q, k, v, d_o, mask=mask)
     _, _, _, dm, _ = oracle.attention_backward(q, k, v, d_o, mask=mask, want_dmask=True)
     np.testing.assert_allclose(dm, dm_t, rtol=0, atol=1e-10)

@@ -95,6 +95,12 @@ int make_params(const TriAttnArgs* a, int need, KParams* p) {
     copy3(p->dvs, a->dv_stride);
     copy3(p->ms, a->mask_stride);
     copy3(p->dms, a->dmask_stride);
+    if (p->dmask != nullptr) {
+        // a stride of 0 over a dimension that has more than one entry: the gradient is summed over it
+        p->dmask_acc = (a->B > 1 && a->dmask_stride[0] == 0) || (a->H > 1 && a->dmask_stride[1] == 0) ||
+                       (a->S > 1 && a->dmask_stride[2] == 0);
+        if (p->dmask_acc && a->mask_dtype != TRI_ATTN_F32) return TRI_ATTN_EDTYPE;
+    }
     p->B = a->B;
     p->H = a->H;
     p->S = a->S;

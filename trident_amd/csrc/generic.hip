@@ -196,8 +196,10 @@ __global__ __launch_bounds__(256) void generic_dq_kernel(const KParams p) {
             if (p.thr8 > 0) dp = dropout_keep(p, bh, row, j) ? dp * p.zscale : 0.f;
             const float ds = pr * (dp - dlt);
             axpy_slice<D>(acc, ds, sK + u * D, part);
-            if (p.dmask && row_ok && j < p.S && part == (u & 3))
-                store_mask_elem(p.dmask, p.mask_dtype, dmrow + j, ds);
+            if (p.dmask && row_ok && j < p.S && part == (u & 3)) {
+                if (p.dmask_acc) unsafeAtomicAdd(static_cast<float*>(p.dmask) + dmrow + j, ds);
+                else store_mask_elem(p.dmask, p.mask_dtype, dmrow + j, ds);
+            }
         }
     }
     if (!row_ok) return;

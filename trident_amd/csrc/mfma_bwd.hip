@@ -38,9 +38,13 @@ __device__ __forceinline__ float mask_at(const void* mask, int64_t off) {
 // transposed LDS reads of the same K tile.
 // RAGGED (4 waves, no mask): S is not a multiple of 128. Rows and keys at or beyond S do not exist: loads clamp
 // their row index to S - 1, keys >= S get probability 0, rows >= S are not stored.
-template <typename T, int D, int NW, bool CAUSAL, int MASK, bool DROPOUT, bool RAGGED = false>
+// DMASK (with a mask): the kernel also writes the mask gradient dS (trident/kernel/attention.py:332-335), each lane four
+// consecutive keys of its row at a time; where the mask is broadcast over a dimension (dmask stride 0) the values are
+// added to the caller's zero-filled fp32 buffer with atomic adds instead.
+template <typename T, int D, int NW, bool CAUSAL, int MASK, bool DROPOUT, bool RAGGED = false, bool DMASK = false>
 __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
     static_assert(!RAGGED || (NW == 4 && MASK == 0), "ragged lengths: 4 waves, no mask");
+    static_assert(!DMASK || MASK != 0, "a mask gradient needs a mask");
     using Tile = SwzTile<D>;
     constexpr int kRows = 32 * NW;
     constexpr int kStages = 4;
@@ -235,6 +239,23 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
             }
 #pragma unroll
             for (int i = 0; i < 16; ++i) ds[i] *= dpt[i] - dlt;
+            if constexpr (DMASK) {
+                const int64_t at = b * p.dms[0] + hd * p.dms[1] + static_cast<int64_t>(qrow) * p.dms[2] + t0 + 32 * kb + 4 * h;
+                if (p.dmask_acc) {
+                    float* dst = static_cast<float*>(p.dmask) + at;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) unsafeAtomicAdd(dst + 8 * (i >> 2) + (i & 3), ds[i]);
+                } else if constexpr (MASK == kMaskF32) {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                        *reinterpret_cast<f32x4*>(static_cast<float*>(p.dmask) + at + 8 * g) = f32x4{ds[4 * g], ds[4 * g + 1], ds[4 * g + 2], ds[4 * g + 3]};
+                } else {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                        *reinterpret_cast<u32x2*>(static_cast<T*>(p.dmask) + at + 8 * g) =
+                            u32x2{Mma<T>::pack2(ds[4 * g], ds[4 * g + 1]), Mma<T>::pack2(ds[4 * g + 2], ds[4 * g + 3])};
+                }
+            }
             u32x4 bop[2];
             bop[0] = pack8<T>(&ds[0]);
             bop[1] = pack8<T>(&ds[8]);
@@ -1504,6 +1525,13 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
 template <typename T, int D, int NW, bool CAUSAL, int MASK>
 int launch_dq_waves(const KParams& p, hipStream_t stream) {
     const dim3 grid(p.B * p.H * (p.S / (32 * NW))), block(64 * NW);
+    if constexpr (MASK != kNoMask) {
+        if (p.dmask != nullptr) {
+            if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dq_kernel<T, D, NW, CAUSAL, MASK, true, false, true>), grid, block, 0, stream, p);
+            else hipLaunchKernelGGL((mfma_dq_kernel<T, D, NW, CAUSAL, MASK, false, false, true>), grid, block, 0, stream, p);
+            return static_cast<int>(hipGetLastError());
+        }
+    }
     if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dq_kernel<T, D, NW, CAUSAL, MASK, true>), grid, block, 0, stream, p);
     else hipLaunchKernelGGL((mfma_dq_kernel<T, D, NW, CAUSAL, MASK, false>), grid, block, 0, stream, p);
     return static_cast<int>(hipGetLastError());

@@ -54,7 +54,7 @@ bool mfma_supported(int which, int dtype, const KParams& p) {
     if (dtype != TRI_ATTN_F16 && dtype != TRI_ATTN_BF16) return false;
     if (p.D != 64 && p.D != 128) return false;
     // lengths that are not multiples of 128 run the 4-wave kernels with boundary handling; those read no mask
-    if (p.S % 128 != 0 && (p.mask != nullptr || p.dmask != nullptr)) return false;
+    if (p.S % 128 != 0 && p.mask != nullptr) return false;
     if (!(p.scale > 0.f)) return false;  // the kernels take row maxima before scaling
     if (!aligned16(p.q) || !aligned16(p.k) || !aligned16(p.v)) return false;
     if (!strides8(p.qs) || !strides8(p.ks) || !strides8(p.vs)) return false;
@@ -77,8 +77,9 @@ bool mfma_supported(int which, int dtype, const KParams& p) {
         case kMfmaDq:
             // (K, V tiles; the phased kernel also stages its Q, dO and O rows that way)
             if (!tile_offsets_fit(p.ks) || !tile_offsets_fit(p.vs) || !tile_offsets_fit(p.qs) || !tile_offsets_fit(p.dos)) return false;
-            // the mask gradient is written by the generic dQ kernel
-            return p.dmask == nullptr && aligned16(p.d_o) && strides8(p.dos) && aligned16(p.dq) && strides8(p.dqs);
+            // the mask gradient leaves in 16-byte (fp32) or 8-byte (16-bit) pieces of four keys
+            if (p.dmask != nullptr && (!aligned16(p.dmask) || (p.dms[0] % 4) || (p.dms[1] % 4) || (p.dms[2] % 4))) return false;
+            return aligned16(p.d_o) && strides8(p.dos) && aligned16(p.dq) && strides8(p.dqs);
         default:
             return false;
     }

@@ -206,7 +206,20 @@ class Attention(torch.autograd.Function):
         delta = torch.empty_like(log2sum) if delta_out is None else delta_out
         full = (num_batches, num_heads, y_size, y_size)
         mask_view = _expand_mask(mask.detach(), full) if mask is not None else None
-        grad_mask_full = torch.empty(full, device=mask.device, dtype=mask.dtype) if want_grad_mask else None
+        # The mask gradient (trident/kernel/attention.py:332-335) in the mask's own shape: a full [B,H,S,S] mask gets
+        # dS written in place; a broadcast mask gets a zero-filled fp32 buffer of its shape that the kernels add to
+        # through strides of 0 (autograd's sum over the broadcast dimensions, without a [B,H,S,S] intermediate).
+        grad_mask_buf = grad_mask_view = None
+        if want_grad_mask:
+            shape4 = (1,) * (4 - mask.dim()) + tuple(mask.shape)
+            if shape4 == full:
+                grad_mask_buf = torch.empty(full, device=mask.device, dtype=mask.dtype)
+                grad_mask_view = grad_mask_buf
+            else:
+                grad_mask_buf = torch.zeros(shape4, device=mask.device, dtype=torch.float32)
+                grad_mask_view = grad_mask_buf.expand(*full)
+                if mask_view.dtype != torch.float32:  # (mask and dmask share one dtype field)
+                    mask_view = _expand_mask(mask.detach().float(), full)
 
         args = _base_args(query, mask_view, dropout_p, is_causal, softmax_scale, seed, offset)
         _fill(args, "q", query, "q_stride")
@@ -219,8 +232,8 @@ class Attention(torch.autograd.Function):
         _fill(args, "dk", grad_key, "dk_stride")
         _fill(args, "dv", grad_value, "dv_stride")
         _fill(args, "delta", delta)
-        if grad_mask_full is not None:
-            _fill(args, "dmask", grad_mask_full, "dmask_stride")
+        if grad_mask_view is not None:
+            _fill(args, "dmask", grad_mask_view, "dmask_stride")
 
         # one call for the three backward launches (trident/operation/attention.py:161-199 launches the
         # delta pre-pass and the backward kernel): the library orders them, and where the dQ kernel can
@@ -230,14 +243,8 @@ class Attention(torch.autograd.Function):
         util.pop_trace()
 
         grad_mask = None
-        if grad_mask_full is not None:
-            grad_mask = grad_mask_full
-            if tuple(mask.shape) != full:
-                # autograd semantics for a broadcast mask: sum over the broadcast dimensions
-                lead = 4 - mask.dim()
-                dims = [i for i in range(4) if i < lead or mask.shape[i - lead] != full[i]]
-                grad_mask = grad_mask_full.float().sum(dim=dims, keepdim=True).to(mask.dtype)
-                grad_mask = grad_mask.reshape(mask.shape)
+        if grad_mask_buf is not None:
+            grad_mask = grad_mask_buf.to(mask.dtype).reshape(mask.shape)
 
         return grad_query, grad_key, grad_value, grad_mask
 
