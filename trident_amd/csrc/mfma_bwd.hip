@@ -1187,9 +1187,12 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
         char* dk0 = static_cast<char*>(p.dk) + (b * p.dks[0] + hd * p.dks[1] + row * p.dks[2] + 32 * DH * member) * 2;
         char* dv0 = static_cast<char*>(p.dv) + (b * p.dvs[0] + hd * p.dvs[1] + row * p.dvs[2] + 32 * DH * member) * 2;
         const float sc = p.scale;
-        Store::run(dk, [sc](float x) { return x * sc; }, patch, dk0, p.dks[2] * 2, lane);
+        // (the lane index taken afresh: the epilogue's per-lane offsets are computed here, not kept across the loop)
+        int elane = threadIdx.x & 63;
+        asm volatile("" : "+v"(elane));
+        Store::run(dk, [sc](float x) { return x * sc; }, patch, dk0, p.dks[2] * 2, elane);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // patch read before it is rewritten
-        Store::run(dv, [](float x) { return x; }, patch, dv0, p.dvs[2] * 2, lane);
+        Store::run(dv, [](float x) { return x; }, patch, dv0, p.dvs[2] * 2, elane);
     }
 }
 
@@ -1206,7 +1209,10 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
 // wave on the matrix pipe and one on the vector ALU. Block r is first read in phase r-1 and last in
 // phase r+2; in phase ph every wave issues its share of block ph+4 and, before the barrier, waits for
 // its share of block ph+2.
-template <typename T, int D, bool CAUSAL>
+// With DROPOUT only -lse / c is folded into the accumulators: dS = P (Z dP - delta) needs delta beside the dropped dP,
+// so the vector phase reads its 16 row values from the block's slot, and draws the keep decisions of its block (one
+// Philox call per lane, shared inside the quad).
+template <typename T, int D, bool CAUSAL, bool DROPOUT = false>
 __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams p) {
     using Tile = SwzTile<D>;
     constexpr int NW = 8;
@@ -1309,8 +1315,17 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
 #pragma unroll
     for (int r = 0; r < 4; ++r) issue_block();
 
-    const int row_off0 = Tile::off(l32, h);
-    const int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
+    int row_off0 = Tile::off(l32, h);
+    int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
+    // Taken afresh at the head of each member's loop: with every register in use, values computed once up here and
+    // needed by only one of the two loops would otherwise be spilled around the other.
+    auto refresh_lane_offsets = [&]() {
+        int l = lane;
+        asm volatile("" : "+v"(l));
+        row_off0 = Tile::off(l & 31, l >> 5);
+        tr_off0 = Tile::tr_off(0, 0, l);
+        tr_off1 = Tile::tr_off(0, 1, l);
+    };
     TRI_WAIT_VMCNT(4 * kLoads);  // K and V have landed
     lds_barrier();
     u32x4 kf[KK], vf[KK];
@@ -1367,7 +1382,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
             if (n == first) {
                 const float* sLse = reinterpret_cast<const float*>(slot_of(rs) + 2 * kHalfBytes);
                 row_lse = sLse[l32];
-                row_delta = sLse[64 + l32];
+                if constexpr (!DROPOUT) row_delta = sLse[64 + l32];
             }
             if (n == 2 * kAccSteps) {
                 const u32x4 zero4 = {0, 0, 0, 0};
@@ -1376,7 +1391,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
                 const uint32_t u2 = Mma<T>::pack2(kFoldUnit, kFoldUnit), u1 = Mma<T>::pack2(kFoldUnit, 0.f);
                 const u32x4 units = h == 0 ? u32x4{u2, u1, 0, 0} : zero4;
                 s = Mma<T>::run(h == 0 ? al : zero4, units, s);
-                dp = Mma<T>::run(h == 0 ? ad : zero4, units, dp);
+                if constexpr (!DROPOUT) dp = Mma<T>::run(h == 0 ? ad : zero4, units, dp);
             }
             if (n < 2 * kAccSteps) {
                 const int m = n % kAccSteps;
@@ -1399,19 +1414,48 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
     using No = std::integral_constant<bool, false>;
 
     // P = exp2(c S') and dS = P dP' of the block whose first row is rb, eight rows at a time, packed as soon as
-    // they are done; only the block on the diagonal pays for the causal comparison
-    auto softmax_backward = [&](auto on_diagonal, int rb) {
+    // they are done; only the block on the diagonal pays for the causal comparison (scores above it become -inf)
+    auto softmax_backward = [&](bool on_diagonal, int rb, int r) {
+        if (on_diagonal) {
+            // a real branch, taken for one block per workgroup; the row base goes through a scalar register the
+            // compiler cannot see through, so that the 16 comparisons are made here and not kept as lane masks
+            // across the whole loop
+            int rbo = rb;
+            asm volatile("" : "+s"(rbo));
+#pragma unroll
+            for (int i = 0; i < 16; ++i) sc_s[i] = key <= rbo + c_row(i, h) ? sc_s[i] : -INFINITY;
+        }
         const f32x16 s = sc_s, dp = sc_dp;
+        const float* sDelta = reinterpret_cast<const float*>(slot_of(r) + 2 * kHalfBytes) + 64;
+        Philox4 mine;  // the block of rows rb + 8 (lane % 4) + 4 h .. +3: this lane's share of the quad's four
+        if constexpr (DROPOUT) mine = dropout_block(p, bh, (rb + 8 * (lane & 3) + 4 * h) >> 2, key >> 2);
 #pragma unroll
         for (int gg = 0; gg < 2; ++gg) {
             float pr[8], ds[8];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int i = 8 * gg + j;
-                float pv = fast_exp2(s[i] * c);
-                if constexpr (decltype(on_diagonal)::value) pv = key <= rb + c_row(i, h) ? pv : 0.f;
-                pr[j] = pv;
-                ds[j] = pv * dp[i];
+            for (int g2 = 0; g2 < 2; ++g2) {
+                const int g = 2 * gg + g2;
+                f32x4 d4 = {0.f, 0.f, 0.f, 0.f};
+                uint32_t dw[4] = {0, 0, 0, 0};
+                if constexpr (DROPOUT) {
+                    d4 = *reinterpret_cast<const f32x4*>(sDelta + 8 * g + 4 * h);
+                    const Philox4 rr = quad_bcast_from(g, mine);  // lane g of the quad generated rows rb + 8 g + 4 h .. +3
+#pragma unroll
+                    for (int bb = 0; bb < 4; ++bb) dw[bb] = (rr.w[bb] >> (8 * (key & 3))) & 0xffu;
+                }
+#pragma unroll
+                for (int bb = 0; bb < 4; ++bb) {
+                    const int i = 4 * g + bb, j = 4 * g2 + bb;
+                    const float pv = fast_exp2(s[i] * c);
+                    if constexpr (DROPOUT) {
+                        const bool keep = static_cast<int>(dw[bb]) >= p.thr8;
+                        pr[j] = keep ? pv * p.zscale : 0.f;
+                        ds[j] = pv * ((keep ? dp[i] * p.zscale : 0.f) - d4[bb]);
+                    } else {
+                        pr[j] = pv;
+                        ds[j] = pv * dp[i];
+                    }
+                }
             }
             cur_p[gg] = pack8<T>(pr);
             cur_s[gg] = pack8<T>(ds);
@@ -1422,8 +1466,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
     auto vector_phase = [&](int r) {
         if (block_on(r)) {
             const int rb = row_first + r * kBR;
-            if (CAUSAL && r == kb) softmax_backward(Yes{}, rb);
-            else softmax_backward(No{}, rb);
+            softmax_backward(CAUSAL && r == kb, rb, r);
         } else {
 #pragma unroll
             for (int g = 0; g < 2; ++g) cur_p[g] = cur_s[g] = u32x4{0, 0, 0, 0};
@@ -1486,6 +1529,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
     }
     const int n_iter = n_blocks / 2;
     if (member == 0) {
+        refresh_lane_offsets();
 #pragma unroll 1
         for (int t = 0; t <= n_iter; ++t) {   // the last round only adds member 1's last block
             const int r = 2 * t;
@@ -1494,6 +1538,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
             run_matrix_phase(2 * t + 1, r);
         }
     } else {
+        refresh_lane_offsets();
         idle_phase(0);
 #pragma unroll 1
         for (int t = 0; t < n_iter; ++t) {
@@ -1515,9 +1560,12 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
         char* dk0 = static_cast<char*>(p.dk) + (b * p.dks[0] + hd * p.dks[1] + row * p.dks[2] + 32 * DH * member) * 2;
         char* dv0 = static_cast<char*>(p.dv) + (b * p.dvs[0] + hd * p.dvs[1] + row * p.dvs[2] + 32 * DH * member) * 2;
         const float sc = p.scale;
-        Store::run(dk, [sc](float x) { return x * sc; }, patch, dk0, p.dks[2] * 2, lane);
+        // (the lane index taken afresh: the epilogue's per-lane offsets are computed here, not kept across the loop)
+        int elane = threadIdx.x & 63;
+        asm volatile("" : "+v"(elane));
+        Store::run(dk, [sc](float x) { return x * sc; }, patch, dk0, p.dks[2] * 2, elane);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // patch read before it is rewritten
-        Store::run(dv, [](float x) { return x; }, patch, dv0, p.dvs[2] * 2, lane);
+        Store::run(dv, [](float x) { return x; }, patch, dv0, p.dvs[2] * 2, elane);
     }
 }
 
@@ -1605,10 +1653,9 @@ int launch_dkdv_dropout(const KParams& p, hipStream_t stream) {
         // for two waves per SIMD, so two waves are paired on each key block of a 128-key workgroup
         const dim3 grid(p.B * p.H * (p.S / kBM)), block(512);
         if constexpr (MASK == kNoMask) {
-            if (p.thr8 <= 0) {
-                hipLaunchKernelGGL((mfma_dkdv_phased_kernel<T, D, CAUSAL>), grid, block, 0, stream, p);
-                return static_cast<int>(hipGetLastError());
-            }
+            if (p.thr8 <= 0) hipLaunchKernelGGL((mfma_dkdv_phased_kernel<T, D, CAUSAL, false>), grid, block, 0, stream, p);
+            else hipLaunchKernelGGL((mfma_dkdv_phased_kernel<T, D, CAUSAL, true>), grid, block, 0, stream, p);
+            return static_cast<int>(hipGetLastError());
         }
         if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dkdv_pair_kernel<T, D, CAUSAL, MASK, true>), grid, block, 0, stream, p);
         else hipLaunchKernelGGL((mfma_dkdv_pair_kernel<T, D, CAUSAL, MASK, false>), grid, block, 0, stream, p);
