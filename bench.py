@@ -72,7 +72,14 @@ class Path:
         ref = ctypes.byref(args)
         # A step is the launch sequence of the operator (tri_attn_fwd, then what tri_attn_bwd launches): where
         # the fused dQ + delta kernel applies, dQ (with delta) and dK/dV; otherwise delta, dK/dV, dQ.
-        self.kernels = [("fwd", lambda: self.check(self.lib.tri_attn_fwd(ref)))]
+        self.kernels = []
+        if mview is not None and self.lib.tri_attn_mask_classes_size(ref) > 0:
+            # the classification of the mask's blocks is part of the step (a caller that reuses a mask pays it once)
+            self.classes = torch.empty(self.lib.tri_attn_mask_classes_size(ref), dtype=torch.uint8, device=dev)
+            args.mask_classes = self.classes.data_ptr()
+            self.kernels.append(("mask_classes", lambda: self.check(self.lib.tri_attn_classify_mask(ref))))
+            self.check(self.lib.tri_attn_classify_mask(ref))
+        self.kernels.append(("fwd", lambda: self.check(self.lib.tri_attn_fwd(ref))))
         if w.backward:
             self.check(self.lib.tri_attn_fwd(ref))
             rc = self.lib.tri_attn_bwd_dq_delta(ref)
@@ -95,7 +102,7 @@ class Path:
         dK/dV is credited its four GEMMs (S, dP, dV, dK) and dQ one (dQ); the S and dP that the
         dQ pass recomputes are not credited. Causal halves everything."""
         unit = self.w.flops() / 4.0  # 1 * B H S^2 D (x 1/2 causal)
-        return {"fwd": 4.0, "bwd_dkdv": 8.0, "bwd_dq": 2.0, "bwd_delta": 0.0}[kernel] * unit
+        return {"fwd": 4.0, "bwd_dkdv": 8.0, "bwd_dq": 2.0, "bwd_delta": 0.0, "mask_classes": 0.0}[kernel] * unit
 
     def algorithmic_bytes(self, kernel):
         B, H, S, D = self.q.shape
@@ -206,7 +213,7 @@ def config_figures(dev, with_cpu):
         pth = Path(wl, dev)
         ms, pk = run_steps(pth, 3 if name == "C5" else 10, 2)
         peak = PEAK_TFLOPS[_dtype_name(wl.dtype)]
-        f = wl.flops() / pk["fwd"] / 1e9
+        f = wl.flops() / (pk["fwd"] + pk.get("mask_classes", 0.0)) / 1e9  # (the classification belongs to the forward)
         row = {"workload": describe(wl), "fwd_tflops": round(f, 2), "fwd_frac_of_peak": round(f / peak, 4),
                "peak_tflops": peak, "kernel_ms": {k: round(v, 5) for k, v in pk.items()}}
         if wl.backward:
@@ -221,6 +228,8 @@ def config_figures(dev, with_cpu):
             logical, unique = 4.0 * B * H * S * S, 4.0 * B * S * S
             row["mask_stream"] = {k: {"logical_GBps": round(logical / pk[k] / 1e6, 1),
                                       "unique_GBps": round(unique / pk[k] / 1e6, 1)} for k in pk if k != "bwd_delta"}
+            lengths = (pth.mask[:, 0, 0] == 0).sum(-1)
+            row["masked_key_fraction"] = round(1.0 - float(lengths.float().mean()) / S, 4)
             row["mask_stream"]["note"] = ("fp32 mask bytes every workgroup asks for (logical: B*H*S*S*4; unique: "
                                           "B*S*S*4, the heads of a batch share it) / kernel duration; HBM peak 8000 GB/s")
         if with_cpu:
@@ -441,7 +450,7 @@ def main():
     peak = PEAK_TFLOPS[dname]
     flops_step = w.flops(w.backward)
     value = flops_step / wall_ms / 1e9
-    fwd_tf = w.flops() / per_kernel["fwd"] / 1e9
+    fwd_tf = w.flops() / (per_kernel["fwd"] + per_kernel.get("mask_classes", 0.0)) / 1e9
 
     dominant = max(per_kernel, key=per_kernel.get)
     dom_flops = path.algorithmic_flops(dominant)

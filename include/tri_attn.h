@@ -47,7 +47,7 @@
 extern "C" {
 #endif
 
-#define TRI_ATTN_ABI_VERSION 2
+#define TRI_ATTN_ABI_VERSION 3
 
 enum {
     TRI_ATTN_F32 = 0,
@@ -107,6 +107,12 @@ typedef struct TriAttnArgs {
     int64_t dmask_stride[4];
 
     void* stream;              /* hipStream_t */
+
+    uint8_t* mask_classes;     /* NULL, or the classes of the mask's 64 x 64 blocks, filled by tri_attn_classify_mask and then
+                                  read by tri_attn_fwd / tri_attn_bwd*: dense [MB][MH][RB][S/64] bytes with MB = B (1 if
+                                  mask_stride[0] == 0), MH = H (1 if mask_stride[1] == 0), RB = S/64 (1 if mask_stride[2] == 0);
+                                  0 = every entry of the block is 0, 1 = every entry is -inf, 2 = anything else.
+                                  Only used where S is a multiple of 128. */
 } TriAttnArgs;
 
 /* ABI version of the loaded library (TRI_ATTN_ABI_VERSION it was built with). */
@@ -158,6 +164,17 @@ int tri_attn_bwd(const TriAttnArgs* args);
  * or threads) race on it and must be serialised by the caller; calls on one stream are ordered. */
 #define TRI_ATTN_NOALLOC_MAX_ROWS (1 << 20)
 int tri_attn_bwd_noalloc(const TriAttnArgs* args);
+
+/* Classifies the 64 x 64 blocks of args->mask into args->mask_classes (see there; caller-allocated, size
+ * tri_attn_mask_classes_size(args) bytes). It has no counterpart in the reference, whose kernel adds every mask
+ * tile as it comes (trident/kernel/attention.py:135-138). With the classes at hand the kernels skip key tiles
+ * that are masked out altogether and do not read mask tiles that are all zero (a key-padding or length mask is
+ * made of such tiles but for one column of blocks); results are unchanged. Reads mask; writes mask_classes.
+ * Returns TRI_ATTN_ENOFUSE (nothing launched) where the classes would not be used: S not a multiple of 128. */
+int tri_attn_classify_mask(const TriAttnArgs* args);
+/* Bytes of mask_classes for these arguments (MB * MH * RB * S/64), 0 where tri_attn_classify_mask does not apply, or a
+ * negative TRI_ATTN_E* code. */
+int64_t tri_attn_mask_classes_size(const TriAttnArgs* args);
 
 /* Which kernel family a call would run, without launching anything (no counterpart in the reference): pass 0 =
  * tri_attn_fwd, 1 = tri_attn_bwd_dkdv, 2 = tri_attn_bwd_dq on these arguments. Returns 1 for the matrix-core (MFMA)

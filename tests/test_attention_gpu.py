@@ -503,6 +503,100 @@ def test_trace_ranges_switch_on(device):
     parity.close(o, o_ref, torch.bfloat16, "traced O")
 
 
+# ------------------------------------------------------------------ mask block classes
+def _block_masks(B, H, S, seed):
+    """Masks made of 64 x 64 blocks of different kinds, and the kinds: 0 all zero, 1 all -inf, 2 mixed."""
+    g = torch.Generator().manual_seed(seed)
+    n = S // 64
+    kinds = torch.randint(0, 3, (B, H, n, n), generator=g)
+    kinds[..., 0] = 2  # (no fully masked row)
+    mask = torch.zeros(B, H, S, S)
+    for idx in torch.nonzero(kinds).tolist():
+        b, h, r, c = idx
+        blk = mask[b, h, 64 * r:64 * r + 64, 64 * c:64 * c + 64]
+        if kinds[b, h, r, c] == 1:
+            blk.fill_(float("-inf"))
+        else:
+            blk.copy_(torch.randn(64, 64, generator=g))
+            blk[::7, ::5] = float("-inf")
+    return mask, kinds
+
+
+def _classes_of(device, mask_view, B, H, S, dtype_code=2):
+    import ctypes
+    from trident_amd import _lib
+    args = _lib.TriAttnArgs()
+    args.struct_size = ctypes.sizeof(args)
+    args.dtype, args.B, args.H, args.S, args.D = dtype_code, B, H, S, 64
+    args.mask, args.mask_dtype = mask_view.data_ptr(), trident.util.dtype(mask_view.dtype)
+    args.mask_stride[:] = list(mask_view.stride())
+    size = _lib.lib().tri_attn_mask_classes_size(ctypes.byref(args))
+    out = torch.full((max(size, 1),), 77, dtype=torch.uint8, device=device)
+    args.mask_classes = out.data_ptr()
+    _lib.check(_lib.lib().tri_attn_classify_mask(ctypes.byref(args)))
+    torch.cuda.synchronize()
+    return out.cpu(), size
+
+
+@pytest.mark.parametrize("mask_dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("mshape", [(2, 3, 384, 384), (2, 1, 384, 384), (1, 1, 1, 384), (1, 3, 384, 384)])
+def test_mask_block_classes(mshape, mask_dtype, device):
+    B, H, S = 2, 3, 384
+    mask, kinds = _block_masks(mshape[0], mshape[1], S, 81)
+    if mshape[2] == 1:
+        mask, kinds = mask[:, :, :1].clone(), kinds[:, :, :1]
+        kinds = torch.where(kinds == 2, torch.tensor(2), kinds)
+        # one row of a mixed block is mixed or, by chance, uniform: recompute from the row itself
+        row = mask[:, :, 0].reshape(mshape[0], mshape[1], S // 64, 64)
+        kinds = torch.where((row == 0).all(-1), 0, torch.where((row == float("-inf")).all(-1), 1, 2))[:, :, None]
+    from trident_amd import operation
+    view = operation._expand_mask(mask.to(mask_dtype).to(device), (B, H, S, S))
+    got, size = _classes_of(device, view, B, H, S)
+    assert size == kinds.numel()
+    assert torch.equal(got[:size].reshape(kinds.shape).long(), kinds)
+
+
+@pytest.mark.parametrize("D,p", [(64, 0.0), (128, 0.0), (64, 0.3)])
+def test_classes_do_not_change_results(D, p, device):
+    """The same calls with and without mask_classes give the same bits: skipped tiles only ever added zeros."""
+    import ctypes
+    from trident_amd import _lib, operation
+    lib = _lib.lib()
+    B, H, S = 2, 2, 512
+    for kind in ("blocks", "lengths"):
+        if kind == "blocks":
+            mask = _block_masks(B, 1, S, 82)[0]
+        else:
+            mask = workloads.length_mask(B, S, torch.Generator().manual_seed(83))[0]
+            mask[1, 0, :, 100:] = float("-inf")   # a batch whose keys stop inside the first 128-key workgroup
+        q, k, v, d_o = [x.to(device) for x in _gen((B, H, S, D), 84, torch.bfloat16)]
+        tm = mask.to(device)
+        outs = []
+        for with_classes in (False, True):
+            o = torch.empty_like(q)
+            lse = torch.empty(B, H, S, device=device)
+            delta = torch.empty_like(lse)
+            dq, dk, dv = [torch.full_like(q, float("nan")) for _ in range(3)]
+            args = operation._base_args(q, operation._expand_mask(tm, (B, H, S, S)), p, False, 1.0 / math.sqrt(D), 5, 0)
+            for name, t, field in [("q", q, "q_stride"), ("k", k, "k_stride"), ("v", v, "v_stride"), ("o", o, "o_stride"),
+                                   ("d_o", d_o, "do_stride"), ("dq", dq, "dq_stride"), ("dk", dk, "dk_stride"),
+                                   ("dv", dv, "dv_stride")]:
+                operation._fill(args, name, t, field)
+            operation._fill(args, "lse", lse)
+            operation._fill(args, "delta", delta)
+            if with_classes:
+                classes = torch.empty(lib.tri_attn_mask_classes_size(ctypes.byref(args)), dtype=torch.uint8, device=device)
+                args.mask_classes = classes.data_ptr()
+                _lib.check(lib.tri_attn_classify_mask(ctypes.byref(args)))
+            _lib.check(lib.tri_attn_fwd(ctypes.byref(args)))
+            _lib.check(lib.tri_attn_bwd(ctypes.byref(args)))
+            torch.cuda.synchronize()
+            outs.append((o, lse, dq, dk, dv))
+        for name, a, b_ in zip(("O", "LSE", "dQ", "dK", "dV"), *outs):
+            assert not torch.isnan(a.float()).any(), (kind, name)
+            assert torch.equal(a, b_), (kind, name)
+
+
 # ------------------------------------------------------------------ full-size properties
 def _abi_full(device, w, q, k, v, d_o, mask):
     """Forward + backward of a whole workload through the operator's two ABI wrappers; returns device tensors."""

@@ -4,8 +4,9 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtrident_attn.so")
+EALIGN = -8
 ENOFUSE = -9  # tri_attn_bwd_dq_delta: no fused kernel for this problem, nothing launched
-ABI_VERSION = 2
+ABI_VERSION = 3
 ESCRATCH = -10  # tri_attn_bwd_noalloc: B*H*S above NOALLOC_MAX_ROWS, nothing launched
 NOALLOC_MAX_ROWS = 1 << 20
 
@@ -49,6 +50,7 @@ class TriAttnArgs(ctypes.Structure):
         ("mask_stride", _i64x4),
         ("dmask_stride", _i64x4),
         ("stream", ctypes.c_void_p),
+        ("mask_classes", ctypes.c_void_p),
     ]
 
 
@@ -88,6 +90,8 @@ EXPORTS = (
     "tri_attn_bwd_noalloc",
     "tri_attn_dropout_mask",
     "tri_attn_uses_matrix_cores",
+    "tri_attn_classify_mask",
+    "tri_attn_mask_classes_size",
     "tri_attn_probe_mfma",
 )
 
@@ -110,10 +114,12 @@ def lib():
         cdll.tri_attn_strerror.restype = ctypes.c_char_p
         cdll.tri_attn_strerror.argtypes = [ctypes.c_int]
         for name in ("tri_attn_fwd", "tri_attn_bwd_delta", "tri_attn_bwd_dkdv", "tri_attn_bwd_dq",
-                     "tri_attn_bwd_dq_delta", "tri_attn_bwd", "tri_attn_bwd_noalloc"):
+                     "tri_attn_bwd_dq_delta", "tri_attn_bwd", "tri_attn_bwd_noalloc", "tri_attn_classify_mask"):
             fn = getattr(cdll, name)
             fn.restype = ctypes.c_int
             fn.argtypes = [ctypes.POINTER(TriAttnArgs)]
+        cdll.tri_attn_mask_classes_size.restype = ctypes.c_int64
+        cdll.tri_attn_mask_classes_size.argtypes = [ctypes.POINTER(TriAttnArgs)]
         cdll.tri_attn_uses_matrix_cores.restype = ctypes.c_int
         cdll.tri_attn_uses_matrix_cores.argtypes = [ctypes.POINTER(TriAttnArgs), ctypes.c_int]
         cdll.tri_attn_dropout_mask.restype = ctypes.c_int

@@ -101,6 +101,14 @@ int make_params(const TriAttnArgs* a, int need, KParams* p) {
                        (a->S > 1 && a->dmask_stride[2] == 0);
         if (p->dmask_acc && a->mask_dtype != TRI_ATTN_F32) return TRI_ATTN_EDTYPE;
     }
+    if (a->mask != nullptr && a->S % 128 == 0) {
+        // layout of the block classes (64 x 64 blocks), broadcast like the mask itself
+        const int64_t cb = a->S / 64, rb = a->mask_stride[2] == 0 ? 1 : cb, mh = a->mask_stride[1] == 0 ? 1 : a->H;
+        p->mcs[2] = rb == 1 ? 0 : cb;
+        p->mcs[1] = mh == 1 ? 0 : rb * cb;
+        p->mcs[0] = a->mask_stride[0] == 0 ? 0 : mh * rb * cb;
+        p->mcls = a->mask_classes;
+    }
     p->B = a->B;
     p->H = a->H;
     p->S = a->S;
@@ -246,6 +254,39 @@ int tri_attn_bwd_noalloc(const TriAttnArgs* args) {
     // every row of delta that dK/dV reads is written first by this call's dQ kernel or delta pre-pass:
     // nothing of the previous call's contents needs clearing
     return tri_attn_bwd(&a);
+}
+
+int64_t tri_attn_mask_classes_size(const TriAttnArgs* args) {
+    if (args == nullptr) return TRI_ATTN_ENULL;
+    if (args->struct_size != sizeof(TriAttnArgs)) return TRI_ATTN_ESIZE;
+    if (args->B <= 0 || args->H <= 0 || args->S <= 0) return TRI_ATTN_ESHAPE;
+    if (args->mask == nullptr || args->S % 128 != 0) return 0;
+    const int64_t cb = args->S / 64, rb = args->mask_stride[2] == 0 ? 1 : cb;
+    return (args->mask_stride[0] == 0 ? 1 : args->B) * (args->mask_stride[1] == 0 ? 1 : args->H) * rb * cb;
+}
+
+int tri_attn_classify_mask(const TriAttnArgs* args) {
+    if (args == nullptr) return TRI_ATTN_ENULL;
+    if (args->struct_size != sizeof(TriAttnArgs)) return TRI_ATTN_ESIZE;
+    if (args->B <= 0 || args->H <= 0 || args->S <= 0) return TRI_ATTN_ESHAPE;
+    if (args->mask == nullptr || args->mask_classes == nullptr) return TRI_ATTN_ENULL;
+    if (args->mask_dtype < TRI_ATTN_F32 || args->mask_dtype > TRI_ATTN_BF16) return TRI_ATTN_EDTYPE;
+    int rc = check_strides(args->mask_stride);
+    if (rc) return rc;
+    if (args->S % 128 != 0) return TRI_ATTN_ENOFUSE;
+    KParams p;
+    memset(&p, 0, sizeof(p));
+    p.mask = args->mask;
+    p.mask_dtype = args->mask_dtype;
+    copy3(p.ms, args->mask_stride);
+    p.B = args->B;
+    p.H = args->H;
+    p.S = args->S;
+    const int64_t cb = args->S / 64, rb = args->mask_stride[2] == 0 ? 1 : cb, mh = args->mask_stride[1] == 0 ? 1 : args->H;
+    p.mcs[2] = rb == 1 ? 0 : cb;
+    p.mcs[1] = mh == 1 ? 0 : rb * cb;
+    p.mcs[0] = args->mask_stride[0] == 0 ? 0 : mh * rb * cb;
+    return launch_classify_mask(p, args->mask_classes, static_cast<hipStream_t>(args->stream));
 }
 
 int tri_attn_uses_matrix_cores(const TriAttnArgs* args, int pass) {

@@ -27,7 +27,9 @@ struct KParams {
     void* dv;
     void* dmask;
     float* delta;
+    const uint8_t* mcls;   // classes of the mask's 64 x 64 blocks or nullptr
     int64_t qs[3], ks[3], vs[3], os[3], dos[3], dqs[3], dks[3], dvs[3], ms[3], dms[3];
+    int64_t mcs[3];        // strides of mcls (bytes) over batch, head, row block; the column-block stride is 1
     int B, H, S, D;
     int causal;
     int mask_dtype;

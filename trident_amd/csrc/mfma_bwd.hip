@@ -94,8 +94,21 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
     for (int db = 0; db < DB; ++db) acc[db] = zero16();
 
     const int num_key_tiles = (p.S + kBN - 1) / kBN;
-    const int n_tiles = CAUSAL ? min((q0 + kRows) / kBN, num_key_tiles) : num_key_tiles;  // tiles the workgroup streams
-    const int my_tiles = CAUSAL ? min((wrow0 + 31) / kBN + 1, n_tiles) : n_tiles;         // tiles with keys visible to this wave
+    int n_tiles = CAUSAL ? min((q0 + kRows) / kBN, num_key_tiles) : num_key_tiles;  // tiles the workgroup streams
+    int my_tiles = CAUSAL ? min((wrow0 + 31) / kBN + 1, n_tiles) : n_tiles;         // tiles with keys visible to this wave
+    // With the classes of the mask's blocks at hand: key tiles behind the last one that is not masked out altogether
+    // are not streamed, and tiles whose mask is all zero over the workgroup's rows are not read.
+    uint64_t zero_tiles = 0;
+    if constexpr (MASK != kNoMask) {
+        if (p.mcls != nullptr && n_tiles <= 64) {
+            const TileClasses tc = tile_classes(p.mcls + b * p.mcs[0] + hd * p.mcs[1] + (q0 / 64) * p.mcs[2], 1, n_tiles,
+                                                kRows / 64, p.mcs[2], lane);
+            zero_tiles = tc.zero;
+            n_tiles = tc.active ? 64 - __builtin_clzll(tc.active) : 1;
+            my_tiles = n_tiles;
+        }
+    }
+    auto mask_is_zero = [&](int t) { return MASK != kNoMask && ((zero_tiles >> t) & 1) != 0; };
 
     int src_off[kBlocksPerWave];
 #pragma unroll
@@ -120,8 +133,9 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
         }
     };
     char* mask_lds = smem + kStages * kStageBytes + wave * kMaskBytes;
-    auto issue_mask = [&](int t) {  // mask block of tile t -> this wave's region
+    auto issue_mask = [&](int t) {  // mask block of tile t -> this wave's region, unless it is all zero
         if constexpr (kMaskViaLds) {
+            if (mask_is_zero(t)) return;
             const char* src = static_cast<const char*>(p.mask) +
                               (b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(wrow0) * p.ms[2] + t * kBN) * 4;
             int l = lane;
@@ -154,7 +168,8 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
         {
             // with a staged mask, block j must have landed too: only tile j+2 was issued after it
             // (tiles 1 and 2 for j = 0)
-            const int younger = kMaskViaLds && j > 0 ? min(1, max(0, n_tiles - 2 - j)) : min(2, n_tiles - 1 - j);
+            // (a block that is all zero was never requested: then the two youngest tiles are what may be in flight)
+            const int younger = kMaskViaLds && j > 0 && !mask_is_zero(j) ? min(1, max(0, n_tiles - 2 - j)) : min(2, n_tiles - 1 - j);
             if (younger == 2) TRI_WAIT_VMCNT(2 * kBlocksPerWave);
             else if (younger == 1) TRI_WAIT_VMCNT(kBlocksPerWave);
             else TRI_WAIT_VMCNT(0);
@@ -163,12 +178,17 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
         float mk2[kMaskViaLds ? 32 : 1];
         if constexpr (kMaskViaLds) {
             // (a mask excludes the causal variant, so every wave works on every tile)
+            if (mask_is_zero(j)) {
 #pragma unroll
-            for (int g = 0; g < 8; ++g) {
-                const f32x4 v = *reinterpret_cast<const f32x4*>(mask_lds + MaskTile::off(l32, 2 * g + h));
-                mk2[4 * g + 0] = v.x; mk2[4 * g + 1] = v.y; mk2[4 * g + 2] = v.z; mk2[4 * g + 3] = v.w;
+                for (int i = 0; i < 32; ++i) mk2[i] = 0.f;
+            } else {
+#pragma unroll
+                for (int g = 0; g < 8; ++g) {
+                    const f32x4 v = *reinterpret_cast<const f32x4*>(mask_lds + MaskTile::off(l32, 2 * g + h));
+                    mk2[4 * g + 0] = v.x; mk2[4 * g + 1] = v.y; mk2[4 * g + 2] = v.z; mk2[4 * g + 3] = v.w;
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // region read before it is refilled
             }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // region read before it is refilled
             if (j + 1 < n_tiles) issue_mask(j + 1);
         }
         if (j + 3 < n_tiles) issue_tile(j + 3);
@@ -185,9 +205,14 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) mk[i] = mk2[16 * kb + i];
             } else if constexpr (MASK != kNoMask) {
-                const int64_t mrow = b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(qrow) * p.ms[2] + t0 + 32 * kb;
+                if (mask_is_zero(j)) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) mk[i] = mask_at<T, MASK>(p.mask, mrow + c_row(i, h));
+                    for (int i = 0; i < 16; ++i) mk[i] = 0.f;
+                } else {
+                    const int64_t mrow = b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(qrow) * p.ms[2] + t0 + 32 * kb;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) mk[i] = mask_at<T, MASK>(p.mask, mrow + c_row(i, h));
+                }
             }
             u32x4 fr[KK];
 #pragma unroll
@@ -617,9 +642,26 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
         const bool is_g = blk >= Tile::kBlocks;
         src_off[i] = static_cast<int>(Tile::src_off(is_g ? blk - Tile::kBlocks : blk, lane, is_g ? grow_bytes : qrow_bytes));
     }
-    const int t_begin = CAUSAL ? k0 / kBN : 0;                  // first tile with rows that see the workgroup's keys
+    int t_begin = CAUSAL ? k0 / kBN : 0;                        // first tile with rows that see the workgroup's keys
     const int my_begin = CAUSAL ? wkey0 / kBN : 0;              // first tile with rows that see this wave's keys
-    const int n_tiles = (p.S + kBN - 1) / kBN;
+    int n_tiles = (p.S + kBN - 1) / kBN;
+    // With the classes of the mask's blocks at hand: row tiles before the first and behind the last one that is not
+    // masked out altogether over the workgroup's keys are not streamed (keys beyond every length: nothing at all, the
+    // gradients are zero), and tiles whose mask is all zero over the workgroup's keys are not read.
+    uint64_t zero_tiles = 0;
+    if constexpr (MASK != kNoMask) {
+        if (p.mcls != nullptr && n_tiles <= 64) {
+            const TileClasses tc = tile_classes(p.mcls + b * p.mcs[0] + hd * p.mcs[1] + k0 / 64, p.mcs[2], n_tiles, kKeys / 64, 1, lane);
+            zero_tiles = tc.zero;
+            if (tc.active) {
+                t_begin = __builtin_ctzll(tc.active);
+                n_tiles = 64 - __builtin_clzll(tc.active);
+            } else {
+                n_tiles = 0;
+            }
+        }
+    }
+    auto mask_is_zero = [&](int t) { return MASK != kNoMask && ((zero_tiles >> t) & 1) != 0; };
     auto issue_tile = [&](int t) {
         char* stage = smem + (t % kStages) * kStageBytes;
         const bool partial = RAGGED && (t + 1) * kBN > p.S;  // the sequence ends inside this tile
@@ -644,8 +686,9 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
         else lds_direct_load4(lse_base + t * kBN, aux, stage + 2 * Tile::kBytes);
     };
     char* mask_lds = smem + kStages * kStageBytes + wave * MaskTile::kBytes;
-    auto issue_mask = [&](int t) {  // rows of tile t x this wave's keys -> the wave's region
+    auto issue_mask = [&](int t) {  // rows of tile t x this wave's keys -> the wave's region, unless the tile is all zero
         if constexpr (kMaskViaLds) {
+            if (mask_is_zero(t)) return;
             const char* src = static_cast<const char*>(p.mask) +
                               (b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(t) * kBN * p.ms[2] + wkey0) * 4;
             int l = lane;
@@ -656,8 +699,10 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
         }
     };
     // issue order: mask block of the first tile, three tiles, then per tile j: mask j+1, tile j+3
-    issue_mask(t_begin);
-    issue_tile(t_begin);
+    if (t_begin < n_tiles) {
+        issue_mask(t_begin);
+        issue_tile(t_begin);
+    }
     if (t_begin + 1 < n_tiles) issue_tile(t_begin + 1);
     if (t_begin + 2 < n_tiles) issue_tile(t_begin + 2);
     // (the K and V fragments were requested before the tiles, so both latencies overlap)
@@ -674,7 +719,8 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
         {
             // with a staged mask, block j must have landed too: only tile j+2 was issued after it
             // (two tiles after the first block)
-            const int younger = kMaskViaLds && j > t_begin ? min(1, max(0, n_tiles - 2 - j)) : min(2, n_tiles - 1 - j);
+            // (a block that is all zero was never requested: then the two youngest tiles are what may be in flight)
+            const int younger = kMaskViaLds && j > t_begin && !mask_is_zero(j) ? min(1, max(0, n_tiles - 2 - j)) : min(2, n_tiles - 1 - j);
             if (younger == 2) TRI_WAIT_VMCNT(2 * kLoadsPerTile);
             else if (younger == 1) TRI_WAIT_VMCNT(kLoadsPerTile);
             else TRI_WAIT_VMCNT(0);
@@ -683,10 +729,15 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
         float mk2[kMaskViaLds ? 32 : 1];
         if constexpr (kMaskViaLds) {
             // (a mask excludes the causal variant, so every wave works on every tile)
+            if (mask_is_zero(j)) {
 #pragma unroll
-            for (int i = 0; i < 32; ++i)
-                mk2[i] = *reinterpret_cast<const float*>(mask_lds + MaskTile::off(32 * (i >> 4) + c_row(i & 15, h), l32 >> 2) + (l32 & 3) * 4);
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // region read before it is refilled
+                for (int i = 0; i < 32; ++i) mk2[i] = 0.f;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 32; ++i)
+                    mk2[i] = *reinterpret_cast<const float*>(mask_lds + MaskTile::off(32 * (i >> 4) + c_row(i & 15, h), l32 >> 2) + (l32 & 3) * 4);
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // region read before it is refilled
+            }
             if (j + 1 < n_tiles) issue_mask(j + 1);
         }
         if (j + 3 < n_tiles) issue_tile(j + 3);
@@ -707,10 +758,15 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
 #pragma unroll
                 for (int i = 0; i < 16; ++i) mk[i] = qb ? mk2[16 + i] : mk2[i];  // static indices keep it in registers
             } else if constexpr (MASK != kNoMask) {
-                const int64_t mbase = b * p.ms[0] + hd * p.ms[1] + key;
+                if (mask_is_zero(j)) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i)
-                    mk[i] = mask_at<T, MASK>(p.mask, mbase + static_cast<int64_t>(rb + c_row(i, h)) * p.ms[2]);
+                    for (int i = 0; i < 16; ++i) mk[i] = 0.f;
+                } else {
+                    const int64_t mbase = b * p.ms[0] + hd * p.ms[1] + key;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i)
+                        mk[i] = mask_at<T, MASK>(p.mask, mbase + static_cast<int64_t>(rb + c_row(i, h)) * p.ms[2]);
+                }
             }
             const int qoff = 32 * qb * Tile::kRowBytes;
             u32x4 fr[KK];

@@ -285,6 +285,29 @@ __device__ __forceinline__ void map_block_for(const KParams& p, int bid, int num
     else map_block(bid, p.B * p.H, num_tiles, order, bh, tile);
 }
 
+// ---------------------------------------------------------------- mask block classes
+// What the classes of the mask's 64 x 64 blocks (tri_attn_classify_mask; 0 all zero, 1 all -inf, 2 mixed) say about
+// the tiles a workgroup streams: tile t (t < n <= 64) covers `across` blocks that lie `step` bytes apart, the first
+// at first[t * tile_step]. Every lane looks at one tile; the answers are wave-uniform bit masks.
+struct TileClasses {
+    uint64_t zero;    // bit t: every entry of the mask over the workgroup's rows (keys) and tile t is 0: nothing to read
+    uint64_t active;  // bit t: not every entry is -inf: the tile contributes
+};
+__device__ __forceinline__ TileClasses tile_classes(const uint8_t* first, int64_t tile_step, int n, int across, int64_t step, int lane) {
+    bool all_zero = lane < n, all_ninf = true;
+    if (lane < n) {
+        for (int i = 0; i < across; ++i) {
+            const int c = first[lane * tile_step + i * step];
+            all_zero &= c == 0;
+            all_ninf &= c == 1;
+        }
+    }
+    TileClasses r;
+    r.zero = __builtin_amdgcn_ballot_w64(all_zero);
+    r.active = __builtin_amdgcn_ballot_w64(lane < n && !all_ninf);
+    return r;
+}
+
 // ---------------------------------------------------------------- coalesced epilogue
 // A wave holds NB transposed C tiles: lane = output row (l32, two lanes per row), 16 registers per
 // tile = 4 groups of 4 consecutive columns. Stored straight from registers, every store instruction

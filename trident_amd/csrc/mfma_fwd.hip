@@ -99,14 +99,29 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
         my_tiles = CAUSAL ? min((wrow0 + 31) / kBN + 1, n_tiles) : n_tiles;       // tiles this wave has visible keys in
     };
     set_item();
+    // With the classes of the mask's blocks at hand (tri_attn_classify_mask): key tiles behind the last one that is not
+    // masked out altogether are not streamed at all, and tiles whose mask is all zero over the workgroup's rows are not
+    // read (a key-padding or length mask is all zero but for one column of blocks).
+    uint64_t zero_tiles = 0;
+    if constexpr (MASK != kNoMask) {
+        if (p.mcls != nullptr && n_tiles <= 64) {
+            const TileClasses tc = tile_classes(p.mcls + b * p.mcs[0] + hd * p.mcs[1] + (qt * kBM / 64) * p.mcs[2], 1, n_tiles,
+                                                kBM / 64, p.mcs[2], lane);
+            zero_tiles = tc.zero;
+            n_tiles = tc.active ? 64 - __builtin_clzll(tc.active) : 1;  // (fully masked rows still run one tile: NaN like softmax)
+            my_tiles = n_tiles;
+        }
+    }
+    auto mask_is_zero = [&](int t) { return MASK != kNoMask && ((zero_tiles >> t) & 1) != 0; };
 
     f32x16 oacc[DB];
     float m, l;  // reference exponent (log2 domain, scaled) and this lane's partial sum
     const float c = p.scale_log2;
 
     char* mask_lds = smem + kStages * kStageBytes + wave * kMaskBytes;
-    auto issue_mask = [&](int t) {  // mask block of tile t -> this wave's region (8 LDS-direct loads)
+    auto issue_mask = [&](int t) {  // mask block of tile t -> this wave's region (8 LDS-direct loads), unless it is all zero
         if constexpr (kMaskViaLds) {
+            if (mask_is_zero(t)) return;
             const char* src = static_cast<const char*>(p.mask) +
                               (b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(wrow0) * p.ms[2] + t * kBN) * 4;
             int l = lane;
@@ -192,6 +207,11 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     // additive mask values of this lane's row for tile t, straight from memory
     auto load_mask = [&](int t) {
         if constexpr (MASK != kNoMask && !kMaskViaLds) {
+            if (mask_is_zero(t)) {
+#pragma unroll
+                for (int e = 0; e < 32; ++e) mk[e] = 0.f;
+                return;
+            }
             const int64_t mrow = b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(qrow) * p.ms[2] + t * kBN;
 #pragma unroll
             for (int g = 0; g < 8; ++g) {
@@ -212,14 +232,19 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
         if constexpr (kMaskViaLds) {
             // block t was requested a matrix phase ago and only the newest tile load may be younger
             // (block 0 precedes tile 0, which has landed)
-            if (!first) wait_loads(false, tile_in_flight);
+            if (mask_is_zero(t)) {
 #pragma unroll
-            for (int g = 0; g < 8; ++g) {
-                const f32x4 v = *reinterpret_cast<const f32x4*>(mask_lds + MaskTile::off(l32, 8 * (g >> 2) + 2 * (g & 3) + h));
-                mk[4 * g + 0] = v.x; mk[4 * g + 1] = v.y; mk[4 * g + 2] = v.z; mk[4 * g + 3] = v.w;
+                for (int e = 0; e < 32; ++e) mk[e] = 0.f;
+            } else {
+                if (!first) wait_loads(false, tile_in_flight);
+#pragma unroll
+                for (int g = 0; g < 8; ++g) {
+                    const f32x4 v = *reinterpret_cast<const f32x4*>(mask_lds + MaskTile::off(l32, 8 * (g >> 2) + 2 * (g & 3) + h));
+                    mk[4 * g + 0] = v.x; mk[4 * g + 1] = v.y; mk[4 * g + 2] = v.z; mk[4 * g + 3] = v.w;
+                }
             }
             // the values are in registers: the region can take the next block
-            if (t + 1 < my_tiles) {
+            if (t + 1 < my_tiles && !mask_is_zero(t + 1)) {
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 issue_mask(t + 1);
             }
@@ -450,7 +475,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
         // after the barrier it is visible to every wave, and the partner group changes phase. The
         // fragment reads stay in flight across the barrier: nothing overwrites their slot before the
         // barrier after next.
-        wait_loads(kMaskViaLds && with_s, issued);
+        wait_loads(kMaskViaLds && with_s && !mask_is_zero(j + 1), issued);
         __builtin_amdgcn_sched_barrier(0);
         asm volatile("s_barrier" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);

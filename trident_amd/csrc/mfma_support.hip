@@ -45,7 +45,59 @@ int launch_delta_t(const KParams& p, hipStream_t stream) {
     return static_cast<int>(hipGetLastError());
 }
 
+// Classes of the mask's 64 x 64 blocks. A wave takes 64 rows x 64 lanes x 16 bytes (256 fp32 or 512 16-bit keys):
+// every lane folds its 16 bytes of each row into two flags (something non-zero, something other than -inf), the
+// lanes of a block combine them, and one lane per block writes the class byte. Reads every mask element once.
+template <typename M>
+__global__ __launch_bounds__(256) void classify_mask_kernel(const KParams p, uint8_t* out, int strips, int64_t waves_total) {
+    constexpr int kPerLane = 16 / sizeof(M);          // keys per lane
+    constexpr int kLanesPerBlock = 64 / kPerLane;     // lanes that cover one 64-key block
+    const int lane = threadIdx.x & 63;
+    const int64_t w = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    if (w >= waves_total) return;
+    const int cb = p.S / 64;
+    const int rbn = p.mcs[2] == 0 ? 1 : cb, mhn = p.mcs[1] == 0 ? 1 : p.H;
+    const int strip = static_cast<int>(w % strips);
+    const int rb = static_cast<int>((w / strips) % rbn);
+    const int mh = static_cast<int>((w / strips / rbn) % mhn);
+    const int mb = static_cast<int>(w / strips / rbn / mhn);
+    const int key0 = (strip * 64 + lane) * kPerLane;
+    const bool live = key0 < p.S;
+    const M* src = static_cast<const M*>(p.mask) + mb * p.ms[0] + mh * p.ms[1] + static_cast<int64_t>(rb) * 64 * p.ms[2] + (live ? key0 : 0);
+    bool nonzero = false, finite = false;
+    for (int r = 0; r < 64; ++r) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(src + r * p.ms[2]);
+        const M* e = reinterpret_cast<const M*>(&v);
+#pragma unroll
+        for (int i = 0; i < kPerLane; ++i) {
+            const float x = static_cast<float>(e[i]);
+            nonzero |= !(x == 0.f);
+            finite |= !(x == -INFINITY);
+        }
+    }
+    int flags = (nonzero ? 1 : 0) | (finite ? 2 : 0);
+#pragma unroll
+    for (int d = 1; d < kLanesPerBlock; d <<= 1) flags |= __shfl_xor(flags, d);
+    if (live && lane % kLanesPerBlock == 0) {
+        const int cls = flags == 2 ? kMaskZero : (flags == 1 ? kMaskNegInf : kMaskMixed);  // (only finite, all of it zero) / (only -inf)
+        out[mb * p.mcs[0] + mh * p.mcs[1] + rb * p.mcs[2] + key0 / 64] = static_cast<uint8_t>(cls);
+    }
+}
+
 }  // namespace
+
+int launch_classify_mask(const KParams& p, uint8_t* out, hipStream_t stream) {
+    const int per_lane = p.mask_dtype == TRI_ATTN_F32 ? 4 : 8;
+    if (!aligned16(p.mask) || (p.ms[0] % per_lane) || (p.ms[1] % per_lane) || (p.ms[2] % per_lane)) return TRI_ATTN_EALIGN;
+    const int strips = (p.S + 64 * per_lane - 1) / (64 * per_lane);
+    const int cb = p.S / 64, rbn = p.mcs[2] == 0 ? 1 : cb, mhn = p.mcs[1] == 0 ? 1 : p.H, mbn = p.mcs[0] == 0 ? 1 : p.B;
+    const int64_t waves = static_cast<int64_t>(mbn) * mhn * rbn * strips;
+    const dim3 grid(static_cast<unsigned>((waves + 3) / 4)), block(256);
+    if (p.mask_dtype == TRI_ATTN_F32) hipLaunchKernelGGL((classify_mask_kernel<float>), grid, block, 0, stream, p, out, strips, waves);
+    else if (p.mask_dtype == TRI_ATTN_F16) hipLaunchKernelGGL((classify_mask_kernel<f16_t>), grid, block, 0, stream, p, out, strips, waves);
+    else hipLaunchKernelGGL((classify_mask_kernel<bf16_t>), grid, block, 0, stream, p, out, strips, waves);
+    return static_cast<int>(hipGetLastError());
+}
 
 // 64 rows of a tile must be reachable with an unsigned 32-bit byte offset (2-byte elements)
 static bool tile_offsets_fit(const int64_t* strides) { return strides[2] >= 0 && strides[2] < (int64_t{1} << 24); }

@@ -72,6 +72,41 @@ def _base_args(query, mask, dropout_p, is_causal, softmax_scale, seed, offset):
     return args
 
 
+# Classes of a mask's 64 x 64 blocks (tri_attn_classify_mask), kept per mask tensor: the forward call computes them, the
+# backward call and later calls with the same, unmodified tensor (other layers, other steps) find them here. An entry
+# dies with its tensor (weak reference) and is recomputed when the tensor was written to (its version counter moved).
+_MASK_CLASSES = {}
+
+
+def _mask_classes(mask: torch.Tensor, args):
+    """Sets args.mask_classes for the mask already described in ``args``; returns the tensor to keep alive, or None
+    where the library has no use for classes (nothing is launched then)."""
+    import weakref
+
+    lib = _lib.lib()
+    size = lib.tri_attn_mask_classes_size(ctypes.byref(args))
+    if size <= 0:
+        return None
+    key = id(mask)
+    entry = _MASK_CLASSES.get(key)
+    signature = (mask._version, tuple(mask.shape), mask.stride(), mask.dtype, args.B, args.H, args.S, args.mask)
+    if entry is not None and entry[0]() is mask and entry[1] == signature:
+        classes = entry[2]
+    else:
+        classes = torch.empty(size, dtype=torch.uint8, device=mask.device)
+        args.mask_classes = classes.data_ptr()
+        status = lib.tri_attn_classify_mask(ctypes.byref(args))
+        if status in (_lib.ENOFUSE, _lib.EALIGN):
+            args.mask_classes = None
+            return None
+        _lib.check(status)
+        if len(_MASK_CLASSES) >= 64:
+            _MASK_CLASSES.clear()
+        _MASK_CLASSES[key] = (weakref.ref(mask, lambda _r, k=key: _MASK_CLASSES.pop(k, None)), signature, classes)
+    args.mask_classes = classes.data_ptr()
+    return classes
+
+
 def _expand_mask(mask: torch.Tensor, shape):
     """View of the additive mask broadcast to [B,H,S,S] (stride 0 on broadcast dims)."""
     view = mask
@@ -182,6 +217,7 @@ class Attention(torch.autograd.Function):
         _fill(args, "v", value, "v_stride")
         _fill(args, "o", output, "o_stride")
         _fill(args, "lse", log2sum)
+        classes = _mask_classes(mask, args) if mask is not None else None  # (kept alive until the call is enqueued)
 
         util.push_trace("kernel.Attention.forward")
         _lib.check(lib.tri_attn_fwd(ctypes.byref(args)))
@@ -234,6 +270,8 @@ class Attention(torch.autograd.Function):
         _fill(args, "delta", delta)
         if grad_mask_view is not None:
             _fill(args, "dmask", grad_mask_view, "dmask_stride")
+        # (the classes describe the mask tensor as the kernels see it: not when it was converted to fp32 above)
+        classes = _mask_classes(mask, args) if mask is not None and mask_view.dtype == mask.dtype else None
 
         # one call for the three backward launches (trident/operation/attention.py:161-199 launches the
         # delta pre-pass and the backward kernel): the library orders them, and where the dQ kernel can
