@@ -446,11 +446,12 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
     f32x16 st[2], dpt[2];  // S^T and dP^T of the current tile (two key blocks)
     u32x4 bop[4];          // dS^T of the current tile as B operands
     u32x4 ring[kRing];
-    auto matrix_phase = [&](auto with_dq, int t) {
+    auto matrix_phase = [&](auto with_dq, int t, bool with_scores = true) {
         constexpr int first = decltype(with_dq)::value ? 0 : kDqSteps;
         f32x16 s_new[2] = {zero16(), zero16()}, dp_new[2] = {zero16(), zero16()};
 #pragma unroll
         for (int n = first; n < kSteps; ++n) {
+            if (n >= kDqSteps && !with_scores) break;
             const int slot = (n - first) % kRing;
             const int m = n - kDqSteps;
             if (n < kDqSteps) acc[n % DB] = Mma<T>::run(ring[slot], bop[n / DB], acc[n % DB]);
@@ -536,10 +537,11 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
         __builtin_amdgcn_sched_barrier(0);
         asm volatile("s_barrier" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
-        // ---- matrix phase (a wave's last tile also runs the S^T / dP^T steps, on whatever the next slot
-        // holds: the result is never used)
+        // ---- matrix phase (a wave's last tile has no successor to score; the dropout variant runs the S^T /
+        // dP^T steps all the same, on whatever the next slot holds: leaving them out costs it registers it does
+        // not have, and the result is never used)
         __builtin_amdgcn_s_setprio(2);
-        matrix_phase(Yes{}, t);
+        matrix_phase(Yes{}, t, DROPOUT || t + 1 < my_tiles);
         __builtin_amdgcn_s_setprio(0);
         __builtin_amdgcn_sched_barrier(0);
         lds_barrier();
@@ -1425,7 +1427,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
         const int m = n - 2 * kAccSteps;
         return lds_read16(slot_of(rs) + (m < KK ? 0 : kHalfBytes), row_off0 ^ ((m % KK) << 5));
     };
-    auto matrix_phase = [&](auto with_acc, int ra, int rb, int rs) {
+    auto matrix_phase = [&](auto with_acc, int ra, int rb, int rs, bool own_on = true, bool score_on = true) {
         constexpr int first = decltype(with_acc)::value ? 0 : 2 * kAccSteps;
         f32x16 s = zero16(), dp = zero16();
         // One more MFMA each puts -lse / c and -delta under S and dP (a row's value split into three 16-bit
@@ -1435,6 +1437,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
 #pragma unroll
         for (int n = first; n < kSteps; ++n) {
             const int slot = (n - first) % kRing;
+            if ((n == kAccSteps && !own_on && !score_on) || (n == 2 * kAccSteps && !score_on)) break;
             if (n == first) {
                 const float* sLse = reinterpret_cast<const float*>(slot_of(rs) + 2 * kHalfBytes);
                 row_lse = sLse[l32];
@@ -1559,10 +1562,12 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
     auto run_matrix_phase = [&](int ph, int r) {
         // this phase's loads first, while the ring's first fragments are still on their way (after the MFMAs
         // they cost 1-1.6 % more cycles, between them 23 %)
+        // (the last rounds have no own block to add and no block r + 2 to score: those steps are left out, except
+        // with dropout, where the shorter instruction stream would cost registers the variant does not have)
         issue_block();
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_setprio(2);
-        matrix_phase(Yes{}, clamp_block(r - 1), clamp_block(r), r + 2);
+        matrix_phase(Yes{}, clamp_block(r - 1), clamp_block(r), r + 2, DROPOUT || r < n_blocks, DROPOUT || r + 2 < n_blocks);
         __builtin_amdgcn_s_setprio(0);
         wait_blocks(ph);
         __builtin_amdgcn_sched_barrier(0);

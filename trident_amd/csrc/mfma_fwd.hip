@@ -275,7 +275,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
         const char* stage_n = smem + ((j + 1) % kStages) * kStageBytes;
         return s < pv ? v_frag(stage_j + kKBytes, s) : k_frag(stage_n, s - pv);
     };
-    auto matrix_phase = [&](auto with_pv, auto with_s, int j) {
+    auto matrix_phase = [&](auto with_pv, auto with_s, int j, bool do_s = true) {
         constexpr int pv = decltype(with_pv)::value ? kPvSteps : 0;
         constexpr int total = pv + (decltype(with_s)::value ? kSteps : 0);
         if constexpr (decltype(with_s)::value) {
@@ -284,6 +284,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
         }
 #pragma unroll
         for (int s = 0; s < total; ++s) {
+            if (s >= pv && !do_s) break;
             if (s < pv) {
                 oacc[s % DB] = Mma<T>::run(ring[s % kRing], pb[s / DB], oacc[s % DB]);
                 // row sums of P (every accumulator row gets the same sum over the 16 keys)
@@ -481,13 +482,14 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
         __builtin_amdgcn_sched_barrier(0);
 
         if (active) {
-            // (a wave's last tile also runs the S^T steps, on whatever the next slot holds: the result
-            // is never used, and one instruction stream serves every tile)
+            // (a wave's last tile has no successor to score and leaves the S^T steps out; with dropout it runs
+            // them on whatever the next slot holds, the result is never used: the branch would cost registers
+            // that variant does not have)
             if (with_s) load_mask(j + 1);
             // the few instructions of this phase go first, so that the matrix pipe never waits for an
             // issue slot behind the partner's vector work
             __builtin_amdgcn_s_setprio(2);
-            matrix_phase(Yes{}, Yes{}, j);
+            matrix_phase(Yes{}, Yes{}, j, with_s || DROPOUT);
             __builtin_amdgcn_s_setprio(0);
             if (with_s) take_mask_block(j + 1, false, issued);
         }
