@@ -192,13 +192,9 @@ def test_mask_gradient_on_the_matrix_cores(dtype, mask_dtype, mshape, D, device)
     tq = q.to(device)
     buf = torch.zeros(mshape, device=device, dtype=torch.float32 if mshape != (B, H, S, S) else mask_dtype)
     mview = operation._expand_mask(mask.to(device).to(buf.dtype), (B, H, S, S))
-    args = operation._base_args(tq, mview, 0.0, False, 0.125, 0, 0)
-    for name, field in [("q", "q_stride"), ("k", "k_stride"), ("v", "v_stride"), ("d_o", "do_stride"), ("dq", "dq_stride")]:
-        operation._fill(args, name, tq, field)
     lse = torch.empty(B, H, S, device=device)
-    operation._fill(args, "lse", lse)
-    operation._fill(args, "delta", lse)
-    operation._fill(args, "dmask", buf.expand(B, H, S, S), "dmask_stride")
+    args = operation._make_args(tq, tq, tq, tq, lse, mview, 0.0, False, 0.125, 0, 0, grad_output=tq, grad_query=tq,
+                                grad_mask=buf.expand(B, H, S, S), delta=lse)
     assert _lib.lib().tri_attn_uses_matrix_cores(ctypes.byref(args), 2) == (0 if dtype == torch.float32 else 1)
 
 
@@ -288,13 +284,10 @@ def _assert_kernel_family(q, mask, p, causal, scale, expected):
     import ctypes
     from trident_amd import _lib, operation
     lse = torch.empty(q.shape[:3], device=q.device, dtype=torch.float32)
-    args = operation._base_args(q, None if mask is None else operation._expand_mask(mask, (*q.shape[:3], q.shape[2])),
-                                p, causal, scale, 0, 0)
-    for name, field in [("q", "q_stride"), ("k", "k_stride"), ("v", "v_stride"), ("o", "o_stride"), ("d_o", "do_stride"),
-                        ("dq", "dq_stride"), ("dk", "dk_stride"), ("dv", "dv_stride")]:
-        operation._fill(args, name, q, field)   # (only pointers' alignment and the strides matter)
-    operation._fill(args, "lse", lse)
-    operation._fill(args, "delta", lse)
+    mview = None if mask is None else operation._expand_mask(mask, (*q.shape[:3], q.shape[2]))
+    # (only the pointers' alignment and the strides matter)
+    args = operation._make_args(q, q, q, q, lse, mview, p, causal, scale, 0, 0, grad_output=q, grad_query=q, grad_key=q,
+                                grad_value=q, delta=lse)
     got = [_lib.lib().tri_attn_uses_matrix_cores(ctypes.byref(args), which) for which in (0, 1, 2)]
     assert got == [1 if expected else 0] * 3, got
 
@@ -435,13 +428,8 @@ def test_combined_backward_matches_the_three_calls(S, D, causal, p, device):
     for combined in (False, True):
         delta = torch.full_like(lse, float("nan"))
         dq, dk, dv = [torch.full_like(q, float("nan")) for _ in range(3)]
-        args = operation._base_args(q, None, p, causal, 1.0 / math.sqrt(D), 99 if p > 0 else 0, 0)
-        for name, t, field in [("q", q, "q_stride"), ("k", k, "k_stride"), ("v", v, "v_stride"), ("o", o, "o_stride"),
-                               ("d_o", d_o, "do_stride"), ("dq", dq, "dq_stride"), ("dk", dk, "dk_stride"),
-                               ("dv", dv, "dv_stride")]:
-            operation._fill(args, name, t, field)
-        operation._fill(args, "lse", lse)
-        operation._fill(args, "delta", delta)
+        args = operation._make_args(q, k, v, o, lse, None, p, causal, 1.0 / math.sqrt(D), 99 if p > 0 else 0, 0,
+                                    d_o, dq, dk, dv, None, delta)
         ref = ctypes.byref(args)
         _lib.check(lib.tri_attn_fwd(ref))
         if combined:
@@ -577,13 +565,8 @@ def test_classes_do_not_change_results(D, p, device):
             lse = torch.empty(B, H, S, device=device)
             delta = torch.empty_like(lse)
             dq, dk, dv = [torch.full_like(q, float("nan")) for _ in range(3)]
-            args = operation._base_args(q, operation._expand_mask(tm, (B, H, S, S)), p, False, 1.0 / math.sqrt(D), 5, 0)
-            for name, t, field in [("q", q, "q_stride"), ("k", k, "k_stride"), ("v", v, "v_stride"), ("o", o, "o_stride"),
-                                   ("d_o", d_o, "do_stride"), ("dq", dq, "dq_stride"), ("dk", dk, "dk_stride"),
-                                   ("dv", dv, "dv_stride")]:
-                operation._fill(args, name, t, field)
-            operation._fill(args, "lse", lse)
-            operation._fill(args, "delta", delta)
+            args = operation._make_args(q, k, v, o, lse, operation._expand_mask(tm, (B, H, S, S)), p, False,
+                                        1.0 / math.sqrt(D), 5, 0, d_o, dq, dk, dv, None, delta)
             if with_classes:
                 classes = torch.empty(lib.tri_attn_mask_classes_size(ctypes.byref(args)), dtype=torch.uint8, device=device)
                 args.mask_classes = classes.data_ptr()

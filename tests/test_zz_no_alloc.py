@@ -24,16 +24,9 @@ def _backward(lib, entry, prob, with_delta):
     q, k, v, d_o, o, lse, causal, p = prob
     D = q.shape[-1]
     dq, dk, dv = [torch.full_like(q, float("nan")) for _ in range(3)]
-    args = operation._base_args(q, None, p, causal, 1.0 / math.sqrt(D), 4242 if p > 0 else 0, 1)
-    for name, t, field in [("q", q, "q_stride"), ("k", k, "k_stride"), ("v", v, "v_stride"), ("o", o, "o_stride"),
-                           ("d_o", d_o, "do_stride"), ("dq", dq, "dq_stride"), ("dk", dk, "dk_stride"),
-                           ("dv", dv, "dv_stride")]:
-        operation._fill(args, name, t, field)
-    operation._fill(args, "lse", lse)
-    delta = None
-    if with_delta:
-        delta = torch.empty_like(lse)
-        operation._fill(args, "delta", delta)
+    delta = torch.empty_like(lse) if with_delta else None
+    args = operation._make_args(q, k, v, o, lse, None, p, causal, 1.0 / math.sqrt(D), 4242 if p > 0 else 0, 1,
+                                d_o, dq, dk, dv, None, delta)
     ref = ctypes.byref(args)
     _lib.check(lib.tri_attn_fwd(ref))
     _lib.check(getattr(lib, entry)(ref))

@@ -49,7 +49,7 @@ def scaled_dot_product_attention(
     Computes scaled dot product attention on query, key and value tensors,
     and applying dropout if a probability greater than 0.0 is specified.
     """
-    return operation.Attention.apply(
+    return operation.Attention.call(
         query, key, value, attn_mask, dropout_p, is_causal, 1.0 / math.sqrt(key.shape[-1]), use_accelerator
     )
 
@@ -67,4 +67,4 @@ def attention(
     argument list of operation.Attention.apply without ``use_accelerator``."""
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(key.shape[-1])
-    return operation.Attention.apply(query, key, value, mask, dropout_p, is_causal, softmax_scale, False)
+    return operation.Attention.call(query, key, value, mask, dropout_p, is_causal, softmax_scale, False)

@@ -49,26 +49,37 @@ def _next_seed():
     return seed, offset
 
 
-def _fill(args: _lib.TriAttnArgs, name: str, t: torch.Tensor, stride_field: str = None):
-    setattr(args, name, t.data_ptr())
-    if stride_field is not None:
-        getattr(args, stride_field)[:] = _strides4(t)
+_NO_STRIDES = (0, 0, 0, 0)
 
 
-def _base_args(query, mask, dropout_p, is_causal, softmax_scale, seed, offset):
+def _strides_or_zero(t):
+    if t is None:
+        return _NO_STRIDES
+    return t.stride() if t.shape[-1] != 1 else tuple(_strides4(t))
+
+
+def _make_args(query, key, value, output, log2sum, mask, dropout_p, is_causal, softmax_scale, seed, offset,
+               grad_output=None, grad_query=None, grad_key=None, grad_value=None, grad_mask=None, delta=None):
+    """TriAttnArgs (include/tri_attn.h) for one call, on torch's current stream of the query's device."""
     args = _lib.TriAttnArgs()
-    args.struct_size = ctypes.sizeof(_lib.TriAttnArgs)
-    args.dtype = util.dtype(query.dtype)
-    args.B, args.H, args.S, args.D = query.shape
-    args.is_causal = 1 if is_causal else 0
-    args.softmax_scale = float(softmax_scale)
-    args.dropout_p = float(dropout_p)
-    args.seed = seed
-    args.offset = offset
-    if mask is not None:
-        args.mask_dtype = util.dtype(mask.dtype)
-        _fill(args, "mask", mask, "mask_stride")
-    args.stream = torch.cuda.current_stream(query.device).cuda_stream
+    num_batches, num_heads, y_size, x_size = query.shape
+    _lib.ARGS_PACKER.pack_into(
+        args, 0,
+        _lib.ARGS_PACKER.size, util.dtype(query.dtype), num_batches, num_heads, y_size, x_size,
+        1 if is_causal else 0, 0 if mask is None else util.dtype(mask.dtype), softmax_scale, dropout_p, seed, offset,
+        query.data_ptr(), key.data_ptr(), value.data_ptr(), output.data_ptr(), log2sum.data_ptr(),
+        0 if mask is None else mask.data_ptr(),
+        0 if grad_output is None else grad_output.data_ptr(),
+        0 if grad_query is None else grad_query.data_ptr(),
+        0 if grad_key is None else grad_key.data_ptr(),
+        0 if grad_value is None else grad_value.data_ptr(),
+        0 if grad_mask is None else grad_mask.data_ptr(),
+        0 if delta is None else delta.data_ptr(),
+        *query.stride(), *key.stride(), *value.stride(), *output.stride(),
+        *_strides_or_zero(grad_output), *_strides_or_zero(grad_query), *_strides_or_zero(grad_key),
+        *_strides_or_zero(grad_value), *_strides_or_zero(mask), *_strides_or_zero(grad_mask),
+        torch._C._cuda_getCurrentRawStream(query.device.index), 0,
+    )
     return args
 
 
@@ -118,7 +129,24 @@ def _expand_mask(mask: torch.Tensor, shape):
     return view
 
 
+class _NoGraph:
+    """Stands in for the autograd context when no gradient is asked for."""
+
+    def save_for_backward(self, *tensors):
+        pass
+
+
 class Attention(torch.autograd.Function):
+    @staticmethod
+    def call(query, key, value, mask, dropout_p, is_causal, softmax_scale, use_accelerator):
+        """``apply`` with the same arguments, checks and result; when no input asks for a gradient (or gradients are
+        switched off) the forward runs without autograd's bookkeeping, which a small problem would feel."""
+        if torch.is_grad_enabled() and (
+            query.requires_grad or key.requires_grad or value.requires_grad or (mask is not None and mask.requires_grad)
+        ):
+            return Attention.apply(query, key, value, mask, dropout_p, is_causal, softmax_scale, use_accelerator)
+        return Attention.forward(_NoGraph(), query, key, value, mask, dropout_p, is_causal, softmax_scale, use_accelerator)
+
     @staticmethod
     def forward(ctx: Any, *args: Any, **kwargs: Any):
         query, key, value, mask, dropout_p, is_causal, softmax_scale, use_accelerator = args
@@ -211,12 +239,7 @@ class Attention(torch.autograd.Function):
         log2sum = torch.empty(num_batches, num_heads, y_size, device=query.device, dtype=torch.float32)
         mask_view = _expand_mask(mask.detach(), (num_batches, num_heads, y_size, y_size)) if mask is not None else None
 
-        args = _base_args(query, mask_view, dropout_p, is_causal, softmax_scale, seed, offset)
-        _fill(args, "q", query, "q_stride")
-        _fill(args, "k", key, "k_stride")
-        _fill(args, "v", value, "v_stride")
-        _fill(args, "o", output, "o_stride")
-        _fill(args, "lse", log2sum)
+        args = _make_args(query, key, value, output, log2sum, mask_view, dropout_p, is_causal, softmax_scale, seed, offset)
         classes = _mask_classes(mask, args) if mask is not None else None  # (kept alive until the call is enqueued)
 
         util.push_trace("kernel.Attention.forward")
@@ -257,19 +280,8 @@ class Attention(torch.autograd.Function):
                 if mask_view.dtype != torch.float32:  # (mask and dmask share one dtype field)
                     mask_view = _expand_mask(mask.detach().float(), full)
 
-        args = _base_args(query, mask_view, dropout_p, is_causal, softmax_scale, seed, offset)
-        _fill(args, "q", query, "q_stride")
-        _fill(args, "k", key, "k_stride")
-        _fill(args, "v", value, "v_stride")
-        _fill(args, "o", output, "o_stride")
-        _fill(args, "lse", log2sum)
-        _fill(args, "d_o", grad_output, "do_stride")
-        _fill(args, "dq", grad_query, "dq_stride")
-        _fill(args, "dk", grad_key, "dk_stride")
-        _fill(args, "dv", grad_value, "dv_stride")
-        _fill(args, "delta", delta)
-        if grad_mask_view is not None:
-            _fill(args, "dmask", grad_mask_view, "dmask_stride")
+        args = _make_args(query, key, value, output, log2sum, mask_view, dropout_p, is_causal, softmax_scale, seed, offset,
+                          grad_output, grad_query, grad_key, grad_value, grad_mask_view, delta)
         # (the classes describe the mask tensor as the kernels see it: not when it was converted to fp32 above)
         classes = _mask_classes(mask, args) if mask is not None and mask_view.dtype == mask.dtype else None
 
