@@ -90,6 +90,39 @@ def test_reference_value_errors():
         trident.util.dtype(torch.int8)
 
 
+def test_value_errors_with_and_without_a_graph():
+    """function.scaled_dot_product_attention runs operation.Attention.forward directly when nothing asks for a
+    gradient, and through autograd otherwise: the argument checks are the same code on both ways."""
+    f = trident.function.scaled_dot_product_attention
+    for grad in (False, True):
+        y = torch.zeros(2, 4, 12, 16, requires_grad=grad)
+        with pytest.raises(ValueError, match="Attention supports only for power of 2 size tensors."):
+            f(y, y, y)
+        x = torch.zeros(1, 1, 8, 16, requires_grad=grad)
+        with pytest.raises(RuntimeError, match="GPU only"):
+            f(x, x, x)
+        with torch.no_grad(), pytest.raises(RuntimeError, match="GPU only"):
+            f(x, x, x)
+
+
+def test_argument_packer_matches_the_structure():
+    """_lib.ARGS_PACKER writes TriAttnArgs in one call: every field must land where the ctypes structure (and the
+    header) has it."""
+    from trident_amd import _lib
+    args = _lib.TriAttnArgs()
+    values = [_lib.ARGS_PACKER.size, 2, 3, 5, 7, 11, 1, 0, 0.25, 0.5, 2**63 + 5, 2**40 + 1]
+    values += [1000 + i for i in range(12)] + [2000 + i for i in range(40)] + [77, 88]
+    _lib.ARGS_PACKER.pack_into(args, 0, *values)
+    assert (args.struct_size, args.dtype, args.B, args.H, args.S, args.D, args.is_causal, args.mask_dtype) == tuple(values[:8])
+    assert (args.softmax_scale, args.dropout_p, args.seed, args.offset) == (0.25, 0.5, 2**63 + 5, 2**40 + 1)
+    pointers = ["q", "k", "v", "o", "lse", "mask", "d_o", "dq", "dk", "dv", "dmask", "delta"]
+    assert [getattr(args, n) for n in pointers] == [1000 + i for i in range(12)]
+    strides = ["q_stride", "k_stride", "v_stride", "o_stride", "do_stride", "dq_stride", "dk_stride", "dv_stride",
+               "mask_stride", "dmask_stride"]
+    assert [x for n in strides for x in getattr(args, n)] == [2000 + i for i in range(40)]
+    assert (args.stream, args.mask_classes) == (77, 88)
+
+
 def test_reference_limits_can_be_lifted():
     """config.reference_limits = False: any sequence length and boolean masks get past the argument checks
     (and then stop at the GPU-only check on this host); head sizes stay powers of two."""

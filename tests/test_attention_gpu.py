@@ -236,6 +236,22 @@ def test_explicit_softmax_scale_and_module(device):
     parity.close(o, o_ref, torch.float16, "module")
 
 
+def test_forward_without_a_graph_is_the_same_forward(device):
+    """Inputs that ask for no gradient (and torch.no_grad) skip autograd's bookkeeping: same kernel, same bits, no
+    grad_fn; with a gradient asked for the result carries one."""
+    q, k, v, _ = [x.to(device) for x in _gen((2, 2, 128, 64), 52, torch.bfloat16)]
+    f = trident.function.scaled_dot_product_attention
+    plain = f(q, k, v, is_causal=True)
+    assert plain.grad_fn is None and not plain.requires_grad
+    qg = q.clone().requires_grad_()
+    tracked = f(qg, k, v, is_causal=True)
+    assert tracked.grad_fn is not None
+    with torch.no_grad():
+        quiet = f(qg, k, v, is_causal=True)
+    assert quiet.grad_fn is None
+    assert torch.equal(plain, tracked.detach()) and torch.equal(plain, quiet)
+
+
 # ------------------------------------------------------------------ dropout
 def test_dropout_mask_bits_match_oracle(device):
     from trident_amd import _lib
