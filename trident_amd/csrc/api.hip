@@ -195,6 +195,7 @@ int tri_attn_fwd(const TriAttnArgs* args) {
     if (rc) return rc;
     hipStream_t st = static_cast<hipStream_t>(args->stream);
     if (mfma_supported(kMfmaFwd, args->dtype, p)) return launch_mfma_fwd(args->dtype, p, st);
+    if (mfma32_supported(kMfmaFwd, args->dtype, p)) return launch_mfma32(kMfmaFwd, args->dtype, p, st);
     return launch_generic_any(kGenericFwd, args->dtype, p, st);
 }
 
@@ -295,7 +296,9 @@ int tri_attn_uses_matrix_cores(const TriAttnArgs* args, int pass) {
     KParams p;
     const int rc = make_params(args, pass == 0 ? 1 : (pass == 1 ? 4 : 8), &p);
     if (rc) return rc;
-    return mfma_supported(pass == 0 ? kMfmaFwd : (pass == 1 ? kMfmaDkdv : kMfmaDq), args->dtype, p) ? 1 : 0;
+    const int which = pass == 0 ? kMfmaFwd : (pass == 1 ? kMfmaDkdv : kMfmaDq);
+    if (mfma_supported(which, args->dtype, p)) return 1;
+    return mfma32_supported(which, args->dtype, p) ? 2 : 0;
 }
 
 int tri_attn_dropout_mask(uint64_t seed, uint64_t offset, float dropout_p, uint32_t bh, int32_t row0, int32_t rows,

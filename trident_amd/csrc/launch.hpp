@@ -21,6 +21,11 @@ int launch_mfma_dq(int dtype, const KParams& p, hipStream_t stream, bool with_de
 bool mfma_dq_fuses_delta(const KParams& p);
 int launch_mfma_dkdv(int dtype, const KParams& p, hipStream_t stream);
 int launch_delta(int dtype, const KParams& p, hipStream_t stream);
+
+// mfma32.hip: the fp32 matrix instruction. fp32 / fp16 / bf16 storage, D in {16,32,64,128}, any S, any mask, rows
+// aligned to four elements. `which` is a MfmaKernel.
+bool mfma32_supported(int which, int dtype, const KParams& p);
+int launch_mfma32(int which, int dtype, const KParams& p, hipStream_t stream);
 // Classes of the mask's 64 x 64 blocks (0 all zero, 1 all -inf, 2 mixed) into `out`, laid out as p.mcs says.
 int launch_classify_mask(const KParams& p, uint8_t* out, hipStream_t stream);
 enum MaskClass { kMaskZero = 0, kMaskNegInf = 1, kMaskMixed = 2 };

@@ -1,0 +1,277 @@
+// Attention on the fp32 matrix instruction (v_mfma_f32_32x32x2_f32): fp32 inputs, and every 16-bit problem the
+// 16-bit MFMA kernels do not take (head sizes 16 and 32, masked lengths that are not multiples of 128). Any S >= 1,
+// D in {16, 32, 64, 128}, fp32 / fp16 / bf16 storage, additive mask of any dtype and broadcast, causal mask, dropout.
+// Products and sums are fp32 throughout (the instruction multiplies fp32 exactly), so results agree with the
+// vector-ALU kernels of generic.hip to rounding; those remain for views whose rows are not 4-element aligned.
+//
+// One 32x32x2 step takes 64 cycles of the matrix pipe for a single 4-byte operand per lane and side, so neither LDS
+// bandwidth nor the vector ALU is anywhere near a limit here: the kernels keep it simple. 256 threads = 4 waves; a
+// wave owns 32 rows (queries in forward and dQ, keys in dK/dV) whose operands stay in registers, the other side
+// streams through LDS as fp32 tiles of 32 rows (row stride D + 4 floats: the 16-byte reads of 32 lanes then spread
+// over all banks), converted on the way in, each tile fetched into registers while the previous one is computed on.
+//
+// Operand layouts (lane = 32 h + l32): A[i = l32][k = h], B[k = h][j = l32], C[i = c_row(r, h)][j = l32] for register r.
+// The order in which a product's k index is walked is free as long as both operands agree, so
+//   * S^T = K Q^T takes K from LDS 16 bytes at a time (dims 8 j + 4 h + 0..3 = four steps) against Q registers in
+//     that order, and leaves lane (h, l32) with query l32 and keys c_row(r, h);
+//   * O^T += V^T P^T walks the keys in exactly that order, step r using keys {c_row(r, 0), c_row(r, 1)}: the
+//     probabilities are B operands as they stand, no exchange between lanes.
+#include "common.hpp"
+#include "launch.hpp"
+#include "mfma_common.hpp"
+
+namespace tri {
+namespace {
+
+constexpr int kRowsPerGroup = 128;  // 4 waves x 32 rows
+constexpr int kTile32 = 32;         // streamed rows per LDS tile
+
+__device__ __forceinline__ f32x16 mma32(float a, float b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
+// four consecutive elements as fp32
+__device__ __forceinline__ float4 load4(const float* ptr) { return *reinterpret_cast<const float4*>(ptr); }
+__device__ __forceinline__ float4 load4(const f16_t* ptr) {
+    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+    const h4 v = *reinterpret_cast<const h4*>(ptr);
+    return float4{static_cast<float>(v[0]), static_cast<float>(v[1]), static_cast<float>(v[2]), static_cast<float>(v[3])};
+}
+__device__ __forceinline__ float4 load4(const bf16_t* ptr) {
+    const uint2 w = *reinterpret_cast<const uint2*>(ptr);
+    return float4{__builtin_bit_cast(float, w.x << 16), __builtin_bit_cast(float, w.x & 0xffff0000u),
+                  __builtin_bit_cast(float, w.y << 16), __builtin_bit_cast(float, w.y & 0xffff0000u)};
+}
+__device__ __forceinline__ void store4(float* ptr, float4 v) { *reinterpret_cast<float4*>(ptr) = v; }
+__device__ __forceinline__ void store4(f16_t* ptr, float4 v) {
+    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+    const h4 o = {static_cast<f16_t>(v.x), static_cast<f16_t>(v.y), static_cast<f16_t>(v.z), static_cast<f16_t>(v.w)};
+    *reinterpret_cast<h4*>(ptr) = o;
+}
+__device__ __forceinline__ void store4(bf16_t* ptr, float4 v) {
+    const uint32_t lo = Mma<bf16_t>::pack2(v.x, v.y), hi = Mma<bf16_t>::pack2(v.z, v.w);
+    *reinterpret_cast<uint2*>(ptr) = uint2{lo, hi};
+}
+
+// A 32-row tile of a [S][D] matrix on its way into LDS: fetch() reads this thread's share into registers (rows past
+// S as zeros), commit() writes it to the tile (row stride D + 4 floats).
+template <typename T, int D>
+struct Stage32 {
+    static constexpr int LD = D + 4;
+    static constexpr int CH = D / 4;                      // 4-element pieces per row
+    static constexpr int N = (kTile32 * CH + 255) / 256;  // pieces per thread
+    float4 r[N];
+    __device__ __forceinline__ void fetch(const T* base, int64_t row_stride, int row0, int S) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const int c = threadIdx.x + 256 * i;
+            const int row = row0 + c / CH;
+            const bool ok = (kTile32 * CH % 256 == 0 || c < kTile32 * CH) && row < S;
+            r[i] = ok ? load4(base + row * row_stride + 4 * (c % CH)) : float4{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    __device__ __forceinline__ void commit(float* tile) const {
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const int c = threadIdx.x + 256 * i;
+            if (kTile32 * CH % 256 == 0 || c < kTile32 * CH) store4(tile + (c / CH) * LD + 4 * (c % CH), r[i]);
+        }
+    }
+};
+
+__device__ __forceinline__ uint32_t pick_word(const Philox4& r, int s) {
+    return s == 0 ? r.w[0] : (s == 1 ? r.w[1] : (s == 2 ? r.w[2] : r.w[3]));
+}
+
+// ------------------------------------------------------------------------------------------------ forward
+template <typename T, int D>
+__global__ __launch_bounds__(256, 2) void mfma32_fwd_kernel(const KParams p) {
+    constexpr int LD = D + 4;
+    constexpr int DB = D >= 32 ? D / 32 : 1;  // 32-wide blocks of the head dimension (D = 16: one, half empty)
+    constexpr int KJ = D / 8;
+    __shared__ __attribute__((aligned(16))) float sK[kTile32 * LD];
+    __shared__ __attribute__((aligned(16))) float sV[kTile32 * LD];
+
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
+    int bh, qt;
+    map_block(blockIdx.x, p.B * p.H, (p.S + kRowsPerGroup - 1) / kRowsPerGroup, p.causal ? kHeavyLast : kUniformTiles, &bh, &qt);
+    const int b = bh / p.H, hd = bh % p.H;
+    const int q0 = qt * kRowsPerGroup, wrow0 = q0 + 32 * wave, qrow = wrow0 + l32;
+    const bool row_ok = qrow < p.S;
+    const int qrow_c = row_ok ? qrow : p.S - 1;
+
+    const T* kbase = static_cast<const T*>(p.k) + b * p.ks[0] + hd * p.ks[1];
+    const T* vbase = static_cast<const T*>(p.v) + b * p.vs[0] + hd * p.vs[1];
+    const int64_t mrow = p.mask ? b * p.ms[0] + hd * p.ms[1] + qrow_c * p.ms[2] : 0;
+
+    // this lane's share of its query row: dims 8 j + 4 h + 0..3
+    float qf[D / 2];
+    {
+        const T* qptr = static_cast<const T*>(p.q) + b * p.qs[0] + hd * p.qs[1] + qrow_c * p.qs[2];
+#pragma unroll
+        for (int j = 0; j < KJ; ++j) {
+            const float4 v = load4(qptr + 8 * j + 4 * h);
+            qf[4 * j + 0] = v.x;
+            qf[4 * j + 1] = v.y;
+            qf[4 * j + 2] = v.z;
+            qf[4 * j + 3] = v.w;
+        }
+    }
+    f32x16 oacc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) oacc[db] = zero16();
+    float m = -INFINITY, l = 0.f;
+
+    const int n_keys = p.causal ? min(p.S, q0 + kRowsPerGroup) : p.S;  // keys some row of the workgroup sees
+    const int n_tiles = (n_keys + kTile32 - 1) / kTile32;
+    Stage32<T, D> kst, vst;
+    kst.fetch(kbase, p.ks[2], 0, p.S);
+    vst.fetch(vbase, p.vs[2], 0, p.S);
+    kst.commit(sK);
+    vst.commit(sV);
+    for (int t = 0; t < n_tiles; ++t) {
+        const int k0 = t * kTile32;
+        if (t + 1 < n_tiles) {
+            kst.fetch(kbase, p.ks[2], k0 + kTile32, p.S);
+            vst.fetch(vbase, p.vs[2], k0 + kTile32, p.S);
+        }
+        __syncthreads();
+        if (!(p.causal && k0 > wrow0 + 31)) {  // (a tile wholly above this wave's rows has nothing for it)
+            f32x16 s = zero16();
+#pragma unroll
+            for (int j = 0; j < KJ; ++j) {
+                const float4 kf = *reinterpret_cast<const float4*>(sK + l32 * LD + 8 * j + 4 * h);
+                s = mma32(kf.x, qf[4 * j + 0], s);
+                s = mma32(kf.y, qf[4 * j + 1], s);
+                s = mma32(kf.z, qf[4 * j + 2], s);
+                s = mma32(kf.w, qf[4 * j + 3], s);
+            }
+            // scores in the log2 domain: this lane has query qrow and keys k0 + c_row(i, h)
+            float x[16];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int key = k0 + c_row(i, h);
+                float v = s[i] * p.scale_log2;
+                if (p.mask && key < p.S) v = fmaf(load_mask_elem(p.mask, p.mask_dtype, mrow + key), kLog2e, v);
+                const bool visible = key < p.S && (!p.causal || key <= qrow);
+                x[i] = visible ? v : -INFINITY;
+                mx = fmaxf(mx, x[i]);
+            }
+            mx = max_xor32(mx);
+            const float m_new = fmaxf(m, mx);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            const float alpha = fast_exp2(m - m_use);
+            m = m_new;
+            l *= alpha;  // (each lane sums its own 16 keys of a tile; the two halves meet at the end)
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) oacc[db][i] *= alpha;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                x[i] = fast_exp2(x[i] - m_use);
+                l += x[i];
+            }
+            if (p.thr8 > 0) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    // keys k0 + 8 g + 4 h + 0..3 of row qrow: one word of one generator block
+                    const Philox4 r = dropout_block(p, bh, qrow >> 2, (k0 + 8 * g + 4 * h) >> 2);
+                    const uint32_t word = pick_word(r, qrow & 3);
+#pragma unroll
+                    for (int bb = 0; bb < 4; ++bb) {
+                        const bool keep = static_cast<int>((word >> (8 * bb)) & 0xffu) >= p.thr8;
+                        x[4 * g + bb] = keep ? x[4 * g + bb] * p.zscale : 0.f;
+                    }
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float* vrow = sV + c_row(r, h) * LD + l32;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    const float a = (D >= 32 || l32 < D) ? vrow[32 * db] : 0.f;
+                    oacc[db] = mma32(a, x[r], oacc[db]);
+                }
+            }
+        }
+        __syncthreads();
+        if (t + 1 < n_tiles) {
+            kst.commit(sK);
+            vst.commit(sV);
+        }
+    }
+    l = sum_xor32(l);
+    const float inv = 1.f / l;
+    if (row_ok) {
+        // O^T accumulators: register 4 g + e of block db is dim 32 db + 8 g + 4 h + e of this lane's query
+        T* orow = static_cast<T*>(p.o) + b * p.os[0] + hd * p.os[1] + static_cast<int64_t>(qrow) * p.os[2];
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d = 32 * db + 8 * g + 4 * h;
+                if (D >= 32 || d < D)
+                    store4(orow + d, float4{oacc[db][4 * g + 0] * inv, oacc[db][4 * g + 1] * inv, oacc[db][4 * g + 2] * inv,
+                                            oacc[db][4 * g + 3] * inv});
+            }
+        if (h == 0) p.lse[static_cast<int64_t>(bh) * p.S + qrow] = m + fast_log2(l);
+    }
+}
+
+template <typename T, int D>
+int launch32(int which, const KParams& p, hipStream_t stream) {
+    const int64_t groups = static_cast<int64_t>((p.S + kRowsPerGroup - 1) / kRowsPerGroup) * p.B * p.H;
+    if (groups > 2147483647LL) return TRI_ATTN_ESHAPE;
+    const dim3 grid(static_cast<unsigned>(groups)), block(256);
+    switch (which) {
+        case kMfmaFwd:
+            hipLaunchKernelGGL((mfma32_fwd_kernel<T, D>), grid, block, 0, stream, p);
+            break;
+        default:
+            return TRI_ATTN_ESHAPE;
+    }
+    return static_cast<int>(hipGetLastError());
+}
+
+template <typename T>
+int launch32_d(int which, const KParams& p, hipStream_t stream) {
+    switch (p.D) {
+        case 16: return launch32<T, 16>(which, p, stream);
+        case 32: return launch32<T, 32>(which, p, stream);
+        case 64: return launch32<T, 64>(which, p, stream);
+        case 128: return launch32<T, 128>(which, p, stream);
+        default: return TRI_ATTN_ESHAPE;
+    }
+}
+
+bool rows4(const void* ptr, const int64_t* s, int elem_bytes) {
+    return reinterpret_cast<uintptr_t>(ptr) % (4 * elem_bytes) == 0 && s[0] % 4 == 0 && s[1] % 4 == 0 && s[2] % 4 == 0;
+}
+
+}  // namespace
+
+bool mfma32_supported(int which, int dtype, const KParams& p) {
+    if (dtype < TRI_ATTN_F32 || dtype > TRI_ATTN_BF16) return false;
+    if (p.D != 16 && p.D != 32 && p.D != 64 && p.D != 128) return false;
+    const int eb = dtype == TRI_ATTN_F32 ? 4 : 2;
+    // rows are read and written four elements at a time
+    if (!rows4(p.q, p.qs, eb) || !rows4(p.k, p.ks, eb) || !rows4(p.v, p.vs, eb)) return false;
+    switch (which) {
+        case kMfmaFwd: return rows4(p.o, p.os, eb);
+        default: return false;
+    }
+}
+
+int launch_mfma32(int which, int dtype, const KParams& p, hipStream_t stream) {
+    switch (dtype) {
+        case TRI_ATTN_F32: return launch32_d<float>(which, p, stream);
+        case TRI_ATTN_F16: return launch32_d<f16_t>(which, p, stream);
+        case TRI_ATTN_BF16: return launch32_d<bf16_t>(which, p, stream);
+        default: return TRI_ATTN_EDTYPE;
+    }
+}
+
+}  // namespace tri
