@@ -195,7 +195,7 @@ def test_mask_gradient_on_the_matrix_cores(dtype, mask_dtype, mshape, D, device)
     lse = torch.empty(B, H, S, device=device)
     args = operation._make_args(tq, tq, tq, tq, lse, mview, 0.0, False, 0.125, 0, 0, grad_output=tq, grad_query=tq,
                                 grad_mask=buf.expand(B, H, S, S), delta=lse)
-    assert _lib.lib().tri_attn_uses_matrix_cores(ctypes.byref(args), 2) == (0 if dtype == torch.float32 else 1)
+    assert _lib.lib().tri_attn_uses_matrix_cores(ctypes.byref(args), 2) == (2 if dtype == torch.float32 else 1)
 
 
 @pytest.mark.parametrize("D", [64, 128])
@@ -405,11 +405,29 @@ def test_any_length_runs_on_the_matrix_cores(dtype, S, D, variant, device):
 
 
 def test_what_the_16_bit_kernels_leave_runs_on_the_fp32_matrix_instruction(device):
-    """Masked problems of other lengths, fp32 problems and small heads: family 2 (v_mfma_f32_32x32x2_f32) where it is
-    built, the vector-ALU kernels (family 0) elsewhere."""
-    _abi_case(device, torch.bfloat16, 200, 64, "mask", 650, matrix_cores=[2, 0, 0])
-    _abi_case(device, torch.float32, 256, 64, "plain", 651, matrix_cores=[2, 0, 0])
-    _abi_case(device, torch.bfloat16, 256, 32, "causal", 652, matrix_cores=[2, 0, 0])
+    """Masked problems of other lengths, fp32 problems and small heads: family 2 (v_mfma_f32_32x32x2_f32) in all
+    three passes."""
+    _abi_case(device, torch.bfloat16, 200, 64, "mask", 650, matrix_cores=[2, 2, 2])
+    _abi_case(device, torch.float32, 256, 64, "plain", 651, matrix_cores=[2, 2, 2])
+    _abi_case(device, torch.bfloat16, 256, 32, "causal", 652, matrix_cores=[2, 2, 2])
+
+
+@pytest.mark.parametrize("variant", ["plain", "causal", "mask", "mask16", "dropout", "causal+dropout"])
+@pytest.mark.parametrize("dtype,S,D", [(torch.float32, 333, 128), (torch.float32, 200, 64), (torch.float32, 97, 32),
+                                       (torch.float32, 70, 16), (torch.float32, 1, 128), (torch.float32, 512, 128),
+                                       (torch.bfloat16, 130, 16), (torch.float16, 260, 32)])
+def test_fp32_matrix_instruction_kernels(dtype, S, D, variant, device):
+    """The kernels on v_mfma_f32_32x32x2_f32 (forward, dQ, dK/dV; the split dK/dV kernel at D = 128) at every head
+    size, over lengths with a ragged last tile (and one of a single row), three heads, every mask mode and dropout."""
+    if variant == "mask16" and dtype == torch.float32:
+        pytest.skip("a 16-bit mask is a mask of the operand type")
+    _abi_case(device, dtype, S, D, variant, 700 + S + D, batches=2 if S < 300 else 1, heads=3, matrix_cores=[2, 2, 2])
+
+
+def test_fp32_matrix_instruction_masked_16_bit_lengths(device):
+    """16-bit problems the 16-bit kernels leave: a masked length that is no multiple of 128, at D = 64 and 128."""
+    _abi_case(device, torch.bfloat16, 200, 128, "mask", 760, heads=3, matrix_cores=[2, 2, 2])
+    _abi_case(device, torch.float16, 72, 64, "mask16", 761, heads=3, matrix_cores=[2, 2, 2])
 
 
 # ------------------------------------------------------------------ tile counts of the phased kernels

@@ -212,6 +212,7 @@ int tri_attn_bwd_dkdv(const TriAttnArgs* args) {
     if (rc) return rc;
     hipStream_t st = static_cast<hipStream_t>(args->stream);
     if (mfma_supported(kMfmaDkdv, args->dtype, p)) return launch_mfma_dkdv(args->dtype, p, st);
+    if (mfma32_supported(kMfmaDkdv, args->dtype, p)) return launch_mfma32(kMfmaDkdv, args->dtype, p, st);
     return launch_generic_any(kGenericDkdv, args->dtype, p, st);
 }
 
@@ -221,6 +222,7 @@ int tri_attn_bwd_dq(const TriAttnArgs* args) {
     if (rc) return rc;
     hipStream_t st = static_cast<hipStream_t>(args->stream);
     if (mfma_supported(kMfmaDq, args->dtype, p)) return launch_mfma_dq(args->dtype, p, st);
+    if (mfma32_supported(kMfmaDq, args->dtype, p)) return launch_mfma32(kMfmaDq, args->dtype, p, st);
     return launch_generic_any(kGenericDq, args->dtype, p, st);
 }
 

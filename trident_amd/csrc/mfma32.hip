@@ -221,6 +221,486 @@ __global__ __launch_bounds__(256, 2) void mfma32_fwd_kernel(const KParams p) {
     }
 }
 
+// ------------------------------------------------------------------------------------------------ dQ (and dMask)
+// Same data flow as the forward kernel: S^T = K Q^T and dP^T = V dO^T against the wave's Q and dO rows in registers,
+// P and dS on the vector ALU (this lane: its query, 16 keys), dQ^T += K^T dS^T walking the keys in accumulator order.
+template <typename T, int D>
+__global__ __launch_bounds__(256, D == 128 ? 1 : 2) void mfma32_dq_kernel(const KParams p) {
+    constexpr int LD = D + 4;
+    constexpr int DB = D >= 32 ? D / 32 : 1;
+    constexpr int KJ = D / 8;
+    __shared__ __attribute__((aligned(16))) float sK[kTile32 * LD];
+    __shared__ __attribute__((aligned(16))) float sV[kTile32 * LD];
+
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
+    int bh, qt;
+    map_block(blockIdx.x, p.B * p.H, (p.S + kRowsPerGroup - 1) / kRowsPerGroup, p.causal ? kHeavyLast : kUniformTiles, &bh, &qt);
+    const int b = bh / p.H, hd = bh % p.H;
+    const int q0 = qt * kRowsPerGroup, wrow0 = q0 + 32 * wave, qrow = wrow0 + l32;
+    const bool row_ok = qrow < p.S;
+    const int qrow_c = row_ok ? qrow : p.S - 1;
+
+    const T* kbase = static_cast<const T*>(p.k) + b * p.ks[0] + hd * p.ks[1];
+    const T* vbase = static_cast<const T*>(p.v) + b * p.vs[0] + hd * p.vs[1];
+    const int64_t mrow = p.mask ? b * p.ms[0] + hd * p.ms[1] + qrow_c * p.ms[2] : 0;
+    const int64_t dmrow = p.dmask ? b * p.dms[0] + hd * p.dms[1] + qrow_c * p.dms[2] : 0;
+
+    float qf[D / 2], gf[D / 2];
+    {
+        const T* qptr = static_cast<const T*>(p.q) + b * p.qs[0] + hd * p.qs[1] + qrow_c * p.qs[2];
+        const T* gptr = static_cast<const T*>(p.d_o) + b * p.dos[0] + hd * p.dos[1] + qrow_c * p.dos[2];
+#pragma unroll
+        for (int j = 0; j < KJ; ++j) {
+            const float4 v = load4(qptr + 8 * j + 4 * h), g = load4(gptr + 8 * j + 4 * h);
+            qf[4 * j + 0] = v.x;
+            qf[4 * j + 1] = v.y;
+            qf[4 * j + 2] = v.z;
+            qf[4 * j + 3] = v.w;
+            gf[4 * j + 0] = g.x;
+            gf[4 * j + 1] = g.y;
+            gf[4 * j + 2] = g.z;
+            gf[4 * j + 3] = g.w;
+        }
+    }
+    const float lse = p.lse[static_cast<int64_t>(bh) * p.S + qrow_c];
+    const float dlt = p.delta[static_cast<int64_t>(bh) * p.S + qrow_c];
+    f32x16 acc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) acc[db] = zero16();
+
+    const int n_keys = p.causal ? min(p.S, q0 + kRowsPerGroup) : p.S;
+    const int n_tiles = (n_keys + kTile32 - 1) / kTile32;
+    Stage32<T, D> kst, vst;
+    kst.fetch(kbase, p.ks[2], 0, p.S);
+    vst.fetch(vbase, p.vs[2], 0, p.S);
+    kst.commit(sK);
+    vst.commit(sV);
+    for (int t = 0; t < n_tiles; ++t) {
+        const int k0 = t * kTile32;
+        if (t + 1 < n_tiles) {
+            kst.fetch(kbase, p.ks[2], k0 + kTile32, p.S);
+            vst.fetch(vbase, p.vs[2], k0 + kTile32, p.S);
+        }
+        __syncthreads();
+        if (!(p.causal && k0 > wrow0 + 31)) {
+            f32x16 s = zero16(), dp = zero16();
+#pragma unroll
+            for (int j = 0; j < KJ; ++j) {
+                const float4 kf = *reinterpret_cast<const float4*>(sK + l32 * LD + 8 * j + 4 * h);
+                const float4 vf = *reinterpret_cast<const float4*>(sV + l32 * LD + 8 * j + 4 * h);
+                s = mma32(kf.x, qf[4 * j + 0], s);
+                dp = mma32(vf.x, gf[4 * j + 0], dp);
+                s = mma32(kf.y, qf[4 * j + 1], s);
+                dp = mma32(vf.y, gf[4 * j + 1], dp);
+                s = mma32(kf.z, qf[4 * j + 2], s);
+                dp = mma32(vf.z, gf[4 * j + 2], dp);
+                s = mma32(kf.w, qf[4 * j + 3], s);
+                dp = mma32(vf.w, gf[4 * j + 3], dp);
+            }
+            float ds[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int key = k0 + c_row(i, h);
+                float v = s[i] * p.scale_log2;
+                if (p.mask && key < p.S) v = fmaf(load_mask_elem(p.mask, p.mask_dtype, mrow + key), kLog2e, v);
+                const bool visible = key < p.S && (!p.causal || key <= qrow);
+                ds[i] = visible ? fast_exp2(v - lse) : 0.f;
+            }
+            if (p.thr8 > 0) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const Philox4 r = dropout_block(p, bh, qrow >> 2, (k0 + 8 * g + 4 * h) >> 2);
+                    const uint32_t word = pick_word(r, qrow & 3);
+#pragma unroll
+                    for (int bb = 0; bb < 4; ++bb) {
+                        const bool keep = static_cast<int>((word >> (8 * bb)) & 0xffu) >= p.thr8;
+                        dp[4 * g + bb] = keep ? dp[4 * g + bb] * p.zscale : 0.f;
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) ds[i] *= dp[i] - dlt;
+            if (p.dmask && row_ok) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int key = k0 + c_row(i, h);
+                    if (key < p.S) {
+                        if (p.dmask_acc) unsafeAtomicAdd(static_cast<float*>(p.dmask) + dmrow + key, ds[i]);
+                        else store_mask_elem(p.dmask, p.mask_dtype, dmrow + key, ds[i]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float* krow = sK + c_row(r, h) * LD + l32;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    const float a = (D >= 32 || l32 < D) ? krow[32 * db] : 0.f;
+                    acc[db] = mma32(a, ds[r], acc[db]);
+                }
+            }
+        }
+        __syncthreads();
+        if (t + 1 < n_tiles) {
+            kst.commit(sK);
+            vst.commit(sV);
+        }
+    }
+    if (row_ok) {
+        T* dqrow = static_cast<T*>(p.dq) + b * p.dqs[0] + hd * p.dqs[1] + static_cast<int64_t>(qrow) * p.dqs[2];
+        const float sc = p.scale;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d = 32 * db + 8 * g + 4 * h;
+                if (D >= 32 || d < D)
+                    store4(dqrow + d, float4{acc[db][4 * g + 0] * sc, acc[db][4 * g + 1] * sc, acc[db][4 * g + 2] * sc,
+                                             acc[db][4 * g + 3] * sc});
+            }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ dK, dV
+// Roles exchanged: a wave owns 32 keys (K and V rows in registers, as B operands), Q and dO stream through LDS in
+// 32-row tiles with their lse and delta. S = Q K^T and dP = dO V^T leave lane (h, l32) with key l32 and rows
+// c_row(r, h); dV^T += dO^T P and dK^T += Q^T dS walk the rows in that order.
+template <typename T, int D>
+__global__ __launch_bounds__(256, D >= 64 ? 1 : 2) void mfma32_dkdv_kernel(const KParams p) {
+    constexpr int LD = D + 4;
+    constexpr int DB = D >= 32 ? D / 32 : 1;
+    constexpr int KJ = D / 8;
+    __shared__ __attribute__((aligned(16))) float sQ[kTile32 * LD];
+    __shared__ __attribute__((aligned(16))) float sG[kTile32 * LD];
+    __shared__ float sLse[kTile32];
+    __shared__ float sDelta[kTile32];
+
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
+    int bh, kt;
+    map_block(blockIdx.x, p.B * p.H, (p.S + kRowsPerGroup - 1) / kRowsPerGroup, p.causal ? kHeavyFirst : kUniformTiles, &bh, &kt);
+    const int b = bh / p.H, hd = bh % p.H;
+    const int g0 = kt * kRowsPerGroup, wkey0 = g0 + 32 * wave, key = wkey0 + l32;
+    const bool key_ok = key < p.S;
+    const int key_c = key_ok ? key : p.S - 1;
+
+    const T* qbase = static_cast<const T*>(p.q) + b * p.qs[0] + hd * p.qs[1];
+    const T* gbase = static_cast<const T*>(p.d_o) + b * p.dos[0] + hd * p.dos[1];
+    const float* lse_base = p.lse + static_cast<int64_t>(bh) * p.S;
+    const float* delta_base = p.delta + static_cast<int64_t>(bh) * p.S;
+    const int64_t mcol = p.mask ? b * p.ms[0] + hd * p.ms[1] + key_c : 0;
+
+    float kf[D / 2], vf[D / 2];
+    {
+        const T* kptr = static_cast<const T*>(p.k) + b * p.ks[0] + hd * p.ks[1] + key_c * p.ks[2];
+        const T* vptr = static_cast<const T*>(p.v) + b * p.vs[0] + hd * p.vs[1] + key_c * p.vs[2];
+#pragma unroll
+        for (int j = 0; j < KJ; ++j) {
+            const float4 a = load4(kptr + 8 * j + 4 * h), c = load4(vptr + 8 * j + 4 * h);
+            kf[4 * j + 0] = a.x;
+            kf[4 * j + 1] = a.y;
+            kf[4 * j + 2] = a.z;
+            kf[4 * j + 3] = a.w;
+            vf[4 * j + 0] = c.x;
+            vf[4 * j + 1] = c.y;
+            vf[4 * j + 2] = c.z;
+            vf[4 * j + 3] = c.w;
+        }
+    }
+    f32x16 dk[DB], dv[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+        dk[db] = zero16();
+        dv[db] = zero16();
+    }
+
+    const int r_begin = p.causal ? g0 : 0;  // rows above the workgroup's first key see none of its keys
+    const int n_tiles = (p.S - r_begin + kTile32 - 1) / kTile32;
+    Stage32<T, D> qst, gst;
+    float aux = 0.f;  // threads 0-31: lse of a row of the tile, threads 32-63: its delta
+    auto fetch_tile = [&](int r0) {
+        qst.fetch(qbase, p.qs[2], r0, p.S);
+        gst.fetch(gbase, p.dos[2], r0, p.S);
+        if (threadIdx.x < 64) {
+            const int row = r0 + l32;
+            aux = row < p.S ? (h == 0 ? lse_base : delta_base)[row] : 0.f;
+        }
+    };
+    auto commit_tile = [&]() {
+        qst.commit(sQ);
+        gst.commit(sG);
+        if (threadIdx.x < 64) (h == 0 ? sLse : sDelta)[l32] = aux;
+    };
+    fetch_tile(r_begin);
+    commit_tile();
+    for (int t = 0; t < n_tiles; ++t) {
+        const int r0 = r_begin + t * kTile32;
+        if (t + 1 < n_tiles) fetch_tile(r0 + kTile32);
+        __syncthreads();
+        if (!(p.causal && r0 + 31 < wkey0)) {  // (rows wholly above this wave's keys see none of them)
+            f32x16 s = zero16(), dp = zero16();
+#pragma unroll
+            for (int j = 0; j < KJ; ++j) {
+                const float4 qa = *reinterpret_cast<const float4*>(sQ + l32 * LD + 8 * j + 4 * h);
+                const float4 ga = *reinterpret_cast<const float4*>(sG + l32 * LD + 8 * j + 4 * h);
+                s = mma32(qa.x, kf[4 * j + 0], s);
+                dp = mma32(ga.x, vf[4 * j + 0], dp);
+                s = mma32(qa.y, kf[4 * j + 1], s);
+                dp = mma32(ga.y, vf[4 * j + 1], dp);
+                s = mma32(qa.z, kf[4 * j + 2], s);
+                dp = mma32(ga.z, vf[4 * j + 2], dp);
+                s = mma32(qa.w, kf[4 * j + 3], s);
+                dp = mma32(ga.w, vf[4 * j + 3], dp);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // this lane: its key, rows r0 + c_row(i, h)
+            float pr[16], ds[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int row = r0 + c_row(i, h);
+                float v = s[i] * p.scale_log2;
+                if (p.mask && row < p.S) v = fmaf(load_mask_elem(p.mask, p.mask_dtype, mcol + row * p.ms[2]), kLog2e, v);
+                const bool visible = row < p.S && key_ok && (!p.causal || key <= row);
+                pr[i] = visible ? fast_exp2(v - sLse[c_row(i, h)]) : 0.f;
+            }
+            if (p.thr8 > 0) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    // rows r0 + 8 g + 4 h + 0..3 of this key: one byte of each word of one generator block
+                    const Philox4 r = dropout_block(p, bh, (r0 + 8 * g + 4 * h) >> 2, key >> 2);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const bool keep = static_cast<int>((r.w[e] >> (8 * (key & 3))) & 0xffu) >= p.thr8;
+                        const int i = 4 * g + e;
+                        ds[i] = pr[i] * ((keep ? dp[i] * p.zscale : 0.f) - sDelta[c_row(i, h)]);
+                        pr[i] = keep ? pr[i] * p.zscale : 0.f;
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) ds[i] = pr[i] * (dp[i] - sDelta[c_row(i, h)]);
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float* grow = sG + c_row(r, h) * LD + l32;
+                const float* qrow = sQ + c_row(r, h) * LD + l32;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    const bool in = D >= 32 || l32 < D;
+                    dv[db] = mma32(in ? grow[32 * db] : 0.f, pr[r], dv[db]);
+                    dk[db] = mma32(in ? qrow[32 * db] : 0.f, ds[r], dk[db]);
+                }
+                __builtin_amdgcn_sched_barrier(0);  // (operand reads stay next to their use: registers are short)
+            }
+        }
+        __syncthreads();
+        if (t + 1 < n_tiles) commit_tile();
+    }
+    if (key_ok) {
+        T* dkrow = static_cast<T*>(p.dk) + b * p.dks[0] + hd * p.dks[1] + static_cast<int64_t>(key) * p.dks[2];
+        T* dvrow = static_cast<T*>(p.dv) + b * p.dvs[0] + hd * p.dvs[1] + static_cast<int64_t>(key) * p.dvs[2];
+        const float sc = p.scale;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d = 32 * db + 8 * g + 4 * h;
+                if (D >= 32 || d < D) {
+                    store4(dkrow + d, float4{dk[db][4 * g + 0] * sc, dk[db][4 * g + 1] * sc, dk[db][4 * g + 2] * sc,
+                                             dk[db][4 * g + 3] * sc});
+                    store4(dvrow + d, float4{dv[db][4 * g + 0], dv[db][4 * g + 1], dv[db][4 * g + 2], dv[db][4 * g + 3]});
+                }
+            }
+    }
+}
+
+// dK, dV at D = 128: the kernel above would need K and V rows (128 registers) beside dK^T and dV^T (128 more) in one
+// wave. Here a workgroup owns 64 keys whose K and V rows sit in LDS for the whole run (B operands are read from there,
+// 16 bytes per four steps, like the A operands), and the two waves of a key block share its query rows: wave (kb, rh)
+// takes the 32-row tiles 2 u + rh, both accumulate the full head dimension, and at the end the rh = 1 wave hands its
+// accumulators to its partner through LDS.
+template <typename T, int D>
+__global__ __launch_bounds__(256, 1) void mfma32_dkdv_split_kernel(const KParams p) {
+    constexpr int LD = D + 4;
+    constexpr int DB = D / 32;
+    constexpr int KJ = D / 8;
+    constexpr int kKeys = 64;
+    static_assert(D >= 64, "accumulators of two waves must fit into the row tiles' LDS");
+    __shared__ __attribute__((aligned(16))) float sK[kKeys * LD];
+    __shared__ __attribute__((aligned(16))) float sV[kKeys * LD];
+    __shared__ __attribute__((aligned(16))) float sQ[2 * kTile32 * LD];  // tiles 2 u and 2 u + 1
+    __shared__ __attribute__((aligned(16))) float sG[2 * kTile32 * LD];
+    __shared__ float sLse[2 * kTile32];
+    __shared__ float sDelta[2 * kTile32];
+
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int kb = wave & 1, rh = wave >> 1;
+    const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
+    int bh, kt;
+    map_block(blockIdx.x, p.B * p.H, (p.S + kKeys - 1) / kKeys, p.causal ? kHeavyFirst : kUniformTiles, &bh, &kt);
+    const int b = bh / p.H, hd = bh % p.H;
+    const int g0 = kt * kKeys, wkey0 = g0 + 32 * kb, key = wkey0 + l32;
+    const bool key_ok = key < p.S;
+    const int key_c = key_ok ? key : p.S - 1;
+
+    const T* qbase = static_cast<const T*>(p.q) + b * p.qs[0] + hd * p.qs[1];
+    const T* gbase = static_cast<const T*>(p.d_o) + b * p.dos[0] + hd * p.dos[1];
+    const float* lse_base = p.lse + static_cast<int64_t>(bh) * p.S;
+    const float* delta_base = p.delta + static_cast<int64_t>(bh) * p.S;
+    const int64_t mcol = p.mask ? b * p.ms[0] + hd * p.ms[1] + key_c : 0;
+
+    // two 32-row tiles per fetch (Stage32 twice: rows r0 .. r0 + 31 and r0 + 32 .. r0 + 63)
+    Stage32<T, D> st[2][2];
+    float aux = 0.f;  // threads 0-63: lse of a row of the two tiles, threads 64-127: its delta
+    auto fetch_rows = [&](int r0) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            st[u][0].fetch(qbase, p.qs[2], r0 + kTile32 * u, p.S);
+            st[u][1].fetch(gbase, p.dos[2], r0 + kTile32 * u, p.S);
+        }
+        if (threadIdx.x < 128) {
+            const int row = r0 + (threadIdx.x & 63);
+            aux = row < p.S ? (threadIdx.x < 64 ? lse_base : delta_base)[row] : 0.f;
+        }
+    };
+    auto commit_rows = [&]() {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            st[u][0].commit(sQ + u * kTile32 * LD);
+            st[u][1].commit(sG + u * kTile32 * LD);
+        }
+        if (threadIdx.x < 128) (threadIdx.x < 64 ? sLse : sDelta)[threadIdx.x & 63] = aux;
+    };
+    {
+        // the workgroup's K and V rows (rows past S as zeros), through the same staging registers
+        const T* kbase = static_cast<const T*>(p.k) + b * p.ks[0] + hd * p.ks[1];
+        const T* vbase = static_cast<const T*>(p.v) + b * p.vs[0] + hd * p.vs[1];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            st[u][0].fetch(kbase, p.ks[2], g0 + kTile32 * u, p.S);
+            st[u][1].fetch(vbase, p.vs[2], g0 + kTile32 * u, p.S);
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            st[u][0].commit(sK + u * kTile32 * LD);
+            st[u][1].commit(sV + u * kTile32 * LD);
+        }
+    }
+    f32x16 dk[DB], dv[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+        dk[db] = zero16();
+        dv[db] = zero16();
+    }
+    const int r_begin = p.causal ? g0 : 0;
+    const int n_steps = (p.S - r_begin + 2 * kTile32 - 1) / (2 * kTile32);
+    fetch_rows(r_begin);
+    commit_rows();
+    const float* myK = sK + (32 * kb + l32) * LD + 4 * h;
+    const float* myV = sV + (32 * kb + l32) * LD + 4 * h;
+    const float* tQ = sQ + rh * kTile32 * LD;
+    const float* tG = sG + rh * kTile32 * LD;
+    for (int u = 0; u < n_steps; ++u) {
+        const int r0 = r_begin + (2 * u + rh) * kTile32;  // this wave's tile
+        if (u + 1 < n_steps) fetch_rows(r_begin + (2 * u + 2) * kTile32);
+        __syncthreads();
+        if (r0 < p.S && !(p.causal && r0 + 31 < wkey0)) {
+            f32x16 s = zero16(), dp = zero16();
+#pragma unroll
+            for (int j = 0; j < KJ; ++j) {
+                const float4 qa = *reinterpret_cast<const float4*>(tQ + l32 * LD + 8 * j + 4 * h);
+                const float4 ga = *reinterpret_cast<const float4*>(tG + l32 * LD + 8 * j + 4 * h);
+                const float4 kf = *reinterpret_cast<const float4*>(myK + 8 * j);
+                const float4 vf = *reinterpret_cast<const float4*>(myV + 8 * j);
+                s = mma32(qa.x, kf.x, s);
+                dp = mma32(ga.x, vf.x, dp);
+                s = mma32(qa.y, kf.y, s);
+                dp = mma32(ga.y, vf.y, dp);
+                s = mma32(qa.z, kf.z, s);
+                dp = mma32(ga.z, vf.z, dp);
+                s = mma32(qa.w, kf.w, s);
+                dp = mma32(ga.w, vf.w, dp);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            float pr[16], ds[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int row = r0 + c_row(i, h);
+                float v = s[i] * p.scale_log2;
+                if (p.mask && row < p.S) v = fmaf(load_mask_elem(p.mask, p.mask_dtype, mcol + row * p.ms[2]), kLog2e, v);
+                const bool visible = row < p.S && key_ok && (!p.causal || key <= row);
+                pr[i] = visible ? fast_exp2(v - sLse[kTile32 * rh + c_row(i, h)]) : 0.f;
+            }
+            if (p.thr8 > 0) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const Philox4 r = dropout_block(p, bh, (r0 + 8 * g + 4 * h) >> 2, key >> 2);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const bool keep = static_cast<int>((r.w[e] >> (8 * (key & 3))) & 0xffu) >= p.thr8;
+                        const int i = 4 * g + e;
+                        ds[i] = pr[i] * ((keep ? dp[i] * p.zscale : 0.f) - sDelta[kTile32 * rh + c_row(i, h)]);
+                        pr[i] = keep ? pr[i] * p.zscale : 0.f;
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) ds[i] = pr[i] * (dp[i] - sDelta[kTile32 * rh + c_row(i, h)]);
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float* grow = tG + c_row(r, h) * LD + l32;
+                const float* qrow = tQ + c_row(r, h) * LD + l32;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    dv[db] = mma32(grow[32 * db], pr[r], dv[db]);
+                    dk[db] = mma32(qrow[32 * db], ds[r], dk[db]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        __syncthreads();
+        if (u + 1 < n_steps) commit_rows();
+    }
+    // the rh = 1 waves pass their sums to their partners: 2 DB blocks of 16 registers per lane, laid out so that a
+    // lane's 16-byte pieces are contiguous over the lanes
+    __syncthreads();
+    {
+        float* xch = (kb == 0 ? sQ : sG);  // 2 DB * 16 * 64 floats = 32 KiB at D = 128: inside one pair of row tiles
+        static_assert(2 * DB * 16 * 64 <= 2 * kTile32 * LD, "exchange area");
+        if (rh == 1) {
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    store4(xch + ((2 * db + 0) * 4 + g) * 256 + lane * 4,
+                           float4{dk[db][4 * g + 0], dk[db][4 * g + 1], dk[db][4 * g + 2], dk[db][4 * g + 3]});
+                    store4(xch + ((2 * db + 1) * 4 + g) * 256 + lane * 4,
+                           float4{dv[db][4 * g + 0], dv[db][4 * g + 1], dv[db][4 * g + 2], dv[db][4 * g + 3]});
+                }
+        }
+        __syncthreads();
+        if (rh == 0 && key_ok) {
+            T* dkrow = static_cast<T*>(p.dk) + b * p.dks[0] + hd * p.dks[1] + static_cast<int64_t>(key) * p.dks[2];
+            T* dvrow = static_cast<T*>(p.dv) + b * p.dvs[0] + hd * p.dvs[1] + static_cast<int64_t>(key) * p.dvs[2];
+            const float sc = p.scale;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int d = 32 * db + 8 * g + 4 * h;
+                    const float4 ok = *reinterpret_cast<const float4*>(xch + ((2 * db + 0) * 4 + g) * 256 + lane * 4);
+                    const float4 ov = *reinterpret_cast<const float4*>(xch + ((2 * db + 1) * 4 + g) * 256 + lane * 4);
+                    store4(dkrow + d, float4{(dk[db][4 * g + 0] + ok.x) * sc, (dk[db][4 * g + 1] + ok.y) * sc,
+                                             (dk[db][4 * g + 2] + ok.z) * sc, (dk[db][4 * g + 3] + ok.w) * sc});
+                    store4(dvrow + d, float4{dv[db][4 * g + 0] + ov.x, dv[db][4 * g + 1] + ov.y, dv[db][4 * g + 2] + ov.z,
+                                             dv[db][4 * g + 3] + ov.w});
+                }
+        }
+    }
+}
+
 template <typename T, int D>
 int launch32(int which, const KParams& p, hipStream_t stream) {
     const int64_t groups = static_cast<int64_t>((p.S + kRowsPerGroup - 1) / kRowsPerGroup) * p.B * p.H;
@@ -229,6 +709,18 @@ int launch32(int which, const KParams& p, hipStream_t stream) {
     switch (which) {
         case kMfmaFwd:
             hipLaunchKernelGGL((mfma32_fwd_kernel<T, D>), grid, block, 0, stream, p);
+            break;
+        case kMfmaDq:
+            hipLaunchKernelGGL((mfma32_dq_kernel<T, D>), grid, block, 0, stream, p);
+            break;
+        case kMfmaDkdv:
+            if constexpr (D == 128) {
+                const int64_t groups64 = static_cast<int64_t>((p.S + 63) / 64) * p.B * p.H;
+                if (groups64 > 2147483647LL) return TRI_ATTN_ESHAPE;
+                hipLaunchKernelGGL((mfma32_dkdv_split_kernel<T, D>), dim3(static_cast<unsigned>(groups64)), block, 0, stream, p);
+            } else {
+                hipLaunchKernelGGL((mfma32_dkdv_kernel<T, D>), grid, block, 0, stream, p);
+            }
             break;
         default:
             return TRI_ATTN_ESHAPE;
@@ -261,6 +753,8 @@ bool mfma32_supported(int which, int dtype, const KParams& p) {
     if (!rows4(p.q, p.qs, eb) || !rows4(p.k, p.ks, eb) || !rows4(p.v, p.vs, eb)) return false;
     switch (which) {
         case kMfmaFwd: return rows4(p.o, p.os, eb);
+        case kMfmaDq: return rows4(p.d_o, p.dos, eb) && rows4(p.dq, p.dqs, eb);
+        case kMfmaDkdv: return rows4(p.d_o, p.dos, eb) && rows4(p.dk, p.dks, eb) && rows4(p.dv, p.dvs, eb);
         default: return false;
     }
 }
