@@ -1,7 +1,7 @@
 // Shape-generic attention kernels: any S >= 1, D in {16,32,64,128}, fp32/fp16/bf16 storage,
-// fp32 arithmetic on the vector ALU. They serve fp32 inputs (where the matrix cores would
-// lose the 1e-4 accuracy the fp32 contract asks for) and every shape the MFMA kernels do not
-// take (S not a multiple of their tile, D < 64, unaligned views).
+// fp32 arithmetic on the vector ALU, element-wise loads and stores. They take what neither matrix-core family
+// does: views whose rows are not aligned to four elements (mfma32.hip serves every aligned problem the
+// 16-bit MFMA kernels leave, fp32 inputs among them), and the delta pre-pass of such problems.
 //
 // Work split: a workgroup of 256 threads owns 64 rows (query rows for forward and dQ, key
 // rows for dK/dV); each row is shared by 4 adjacent lanes that each hold D/4 of the head
