@@ -425,7 +425,7 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
-    w = workloads.WORKLOADS[a.workload]
+    w = {**workloads.WORKLOADS, **workloads.EXTRA_WORKLOADS}[a.workload]
     if a.ceiling:
         print(json.dumps({"ceiling": ceiling(dev)}), flush=True)
         return

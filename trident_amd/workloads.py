@@ -44,6 +44,11 @@ WORKLOADS = {
     "C5": Workload("C5", torch.bfloat16, 1, 32, 16384, 128, is_causal=True, dropout_p=0.1, sigma_qkv=0.5, seed=1005),
 }
 
+# Beyond the five benchmark configurations: C3's shape in fp32 (the kernels on the fp32 matrix instruction at a real size).
+EXTRA_WORKLOADS = {
+    "F3": Workload("F3", torch.float32, 2, 16, 4096, 128, is_causal=True, seed=1103),
+}
+
 
 def length_mask(B, S, generator):
     """fp32 additive mask [B,1,S,S]: per batch a length in [S/2, S]; keys >= length are -inf."""
