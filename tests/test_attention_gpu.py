@@ -430,6 +430,37 @@ def test_fp32_matrix_instruction_masked_16_bit_lengths(device):
     _abi_case(device, torch.float16, 72, 64, "mask16", 761, heads=3, matrix_cores=[2, 2, 2])
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_views_that_are_not_four_element_aligned_take_the_vector_alu_kernels(dtype, device):
+    """Rows D + 1 elements apart (and a pointer one element into its buffer): neither matrix-core family reads such
+    rows (16-byte / four-element accesses), the element-wise kernels do."""
+    from trident_amd.operation import Attention
+    B, H, S, D = 1, 3, 150, 64
+    q, k, v, d_o = _gen((B, H, S, D), 790, dtype)
+
+    def odd_view(x):
+        buf = torch.zeros(B, H, S, D + 1, dtype=dtype, device=device).flatten()
+        buf = torch.cat([buf, buf.new_zeros(1)])[1:]          # one element past an aligned address
+        view = buf.view(B, H, S, D + 1)[..., :D]
+        view.copy_(x)
+        return view
+
+    tq, tk, tv, tdo = [odd_view(x) for x in (q, k, v, d_o)]
+    assert tq.stride(2) == D + 1 and tq.stride(3) == 1
+    scale = 1.0 / math.sqrt(D)
+    _assert_kernel_family(tq, None, 0.0, True, scale, [0, 0, 0])
+    o, lse = Attention._forward(tq, tk, tv, None, 0.0, True, scale, 0, 0)
+    dq, dk, dv, _ = Attention._backward(tdo, tq, tk, tv, o, lse, None, scale, 0.0, True, 0, 0, False)
+    kw = dict(is_causal=True, scale=scale)
+    o_ref, _ = parity.oracle_forward(q, k, v, **kw)
+    parity.close(o, o_ref, dtype, "odd view O")
+    dq_r, dk_r, dv_r, _, _ = parity.oracle_backward(q, k, v, d_o, o=o, **kw)
+    _, a_dq, a_dk, a_dv = parity.oracle_abs_sums(q, k, v, d_o, o=o, **kw)
+    parity.close(dq, dq_r, dtype, "odd view dQ", a_dq)
+    parity.close(dk, dk_r, dtype, "odd view dK", a_dk)
+    parity.close(dv, dv_r, dtype, "odd view dV", a_dv)
+
+
 # ------------------------------------------------------------------ tile counts of the phased kernels
 @pytest.mark.parametrize("variant", ["plain", "causal", "causal+dropout"])
 @pytest.mark.parametrize("S,D", [(256, 128), (768, 128), (1280, 128), (768, 64), (1024, 64)])
