@@ -76,11 +76,12 @@ def test_modules_keep_dtype(dtype, device):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("shape,dim", [((5, 7), 1), ((64, 2048), 1), ((9, 2056), 1), ((3, 5000), 1), ((17, 4097), 1),
+@pytest.mark.parametrize("shape,dim", [((5, 7), 1), ((64, 2048), 1), ((9, 2056), 1), ((3, 5000), 1), ((17, 4097), 1), ((3, 20000), 1),
                                        ((300, 33), 0), ((4, 6, 128), 2)])
 def test_softmax_shapes_and_dtypes(shape, dim, dtype, device):
-    """Wave-per-row and workgroup-per-row kernels, 16-byte and per-element accesses (odd lengths), the
-    thread-per-row kernel (dim 0), a contiguous 3-D input along its last dimension."""
+    """Wave-per-row and workgroup-per-row kernels, rows that stay in registers and rows too long for that (two sweeps),
+    16-byte and per-element accesses (odd lengths), the thread-per-row kernel (dim 0), a contiguous 3-D input along
+    its last dimension."""
     x, g = _pair(shape, 10 + shape[-1], dtype)
     _softmax_case(device, x * 3, g, dim, dtype, tag=f"softmax {shape} {dtype}")
 

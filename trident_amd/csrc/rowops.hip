@@ -63,9 +63,12 @@ struct alignas(sizeof(T) * V) Vec {
 };
 
 // ------------------------------------------------------------------ rows with unit stride along x
-// G threads share a row (a wave for short rows, the whole workgroup for long ones). Two sweeps over the row:
-// statistics, then the output; the second sweep finds the row in the L2 it was just read through, so the HBM
-// traffic is one read and one write. V elements per load (16 bytes when the row geometry allows it).
+// G threads share a row (a wave for short rows, the whole workgroup for long ones), V elements per load (16 bytes
+// when the row geometry allows it). A row of up to G * V * kHeld elements is read once, all loads in flight together,
+// and stays in registers between the statistics and the output; a longer row takes two sweeps, the second of which
+// finds the row in the L2 it was just read through. Either way the HBM traffic is one read and one write.
+constexpr int kHeld = 4;  // 16-byte pieces of a row a thread keeps
+
 template <typename T, int V, int G, typename M>
 __global__ __launch_bounds__(256) void softmax_fwd_rows_kernel(const RowParams p) {
     __shared__ Stat part[4];
@@ -77,24 +80,45 @@ __global__ __launch_bounds__(256) void softmax_fwd_rows_kernel(const RowParams p
     const T* in = static_cast<const T*>(p.input) + base;
     T* out = static_cast<T*>(p.output) + base;
     using VT = Vec<T, V>;
-
+    const bool resident = p.x_size <= static_cast<int64_t>(G) * V * kHeld;
+    VT held[kHeld];
+    if (live && resident) {
+#pragma unroll
+        for (int k = 0; k < kHeld; ++k) {
+            const int64_t i = (static_cast<int64_t>(k) * G + t) * V;
+            if (i < p.x_size) held[k] = *reinterpret_cast<const VT*>(in + i);
+        }
+    }
+    // x[e] in the log2 domain, masked positions at -inf
+    auto scores = [&](const VT& v, int64_t i, float (&x)[V]) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+            x[e] = to_f32(v.e[e]) * kLog2e;
+            if (mask_hit<M>(p.mask, base + i + e)) x[e] = -INFINITY;
+        }
+    };
     Stat s{-INFINITY, 0.f};
+    auto absorb = [&](const VT& v, int64_t i) {
+        float x[V];
+        scores(v, i, x);
+        float cm = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < V; ++e) cm = fmaxf(cm, x[e]);
+        const float m_new = fmaxf(s.m, cm), ms = safe(m_new);
+        float acc = s.l * fast_exp2(s.m - ms);
+#pragma unroll
+        for (int e = 0; e < V; ++e) acc += fast_exp2(x[e] - ms);
+        s = Stat{m_new, acc};
+    };
     if (live) {
-        for (int64_t i = static_cast<int64_t>(t) * V; i < p.x_size; i += G * V) {
-            const VT v = *reinterpret_cast<const VT*>(in + i);
-            float x[V];
-            float cm = -INFINITY;
+        if (resident) {
 #pragma unroll
-            for (int e = 0; e < V; ++e) {
-                x[e] = to_f32(v.e[e]) * kLog2e;
-                if (mask_hit<M>(p.mask, base + i + e)) x[e] = -INFINITY;
-                cm = fmaxf(cm, x[e]);
+            for (int k = 0; k < kHeld; ++k) {
+                const int64_t i = (static_cast<int64_t>(k) * G + t) * V;
+                if (i < p.x_size) absorb(held[k], i);
             }
-            const float m_new = fmaxf(s.m, cm), ms = safe(m_new);
-            float acc = s.l * fast_exp2(s.m - ms);
-#pragma unroll
-            for (int e = 0; e < V; ++e) acc += fast_exp2(x[e] - ms);
-            s = Stat{m_new, acc};
+        } else {
+            for (int64_t i = static_cast<int64_t>(t) * V; i < p.x_size; i += G * V) absorb(*reinterpret_cast<const VT*>(in + i), i);
         }
     }
     s = wave_merge(s);
@@ -105,16 +129,22 @@ __global__ __launch_bounds__(256) void softmax_fwd_rows_kernel(const RowParams p
     }
     if (!live) return;
     const float ms = safe(s.m), inv = 1.f / s.l;  // a fully masked row: 0 * inf = NaN, as softmax gives
-    for (int64_t i = static_cast<int64_t>(t) * V; i < p.x_size; i += G * V) {
-        const VT v = *reinterpret_cast<const VT*>(in + i);
+    auto emit = [&](const VT& v, int64_t i) {
+        float x[V];
+        scores(v, i, x);
         VT o;
 #pragma unroll
-        for (int e = 0; e < V; ++e) {
-            float x = to_f32(v.e[e]) * kLog2e;
-            if (mask_hit<M>(p.mask, base + i + e)) x = -INFINITY;
-            o.e[e] = from_f32<T>(fast_exp2(x - ms) * inv);
-        }
+        for (int e = 0; e < V; ++e) o.e[e] = from_f32<T>(fast_exp2(x[e] - ms) * inv);
         *reinterpret_cast<VT*>(out + i) = o;
+    };
+    if (resident) {
+#pragma unroll
+        for (int k = 0; k < kHeld; ++k) {
+            const int64_t i = (static_cast<int64_t>(k) * G + t) * V;
+            if (i < p.x_size) emit(held[k], i);
+        }
+    } else {
+        for (int64_t i = static_cast<int64_t>(t) * V; i < p.x_size; i += G * V) emit(*reinterpret_cast<const VT*>(in + i), i);
     }
 }
 
@@ -130,14 +160,31 @@ __global__ __launch_bounds__(256) void softmax_bwd_rows_kernel(const RowParams p
     const T* g = static_cast<const T*>(p.grad_output) + base;
     T* gi = static_cast<T*>(p.grad_input) + base;
     using VT = Vec<T, V>;
-
-    float delta = 0.f;
-    if (live) {
-        for (int64_t i = static_cast<int64_t>(t) * V; i < p.x_size; i += G * V) {
-            const VT ov = *reinterpret_cast<const VT*>(o + i);
-            const VT gv = *reinterpret_cast<const VT*>(g + i);
+    const bool resident = p.x_size <= static_cast<int64_t>(G) * V * kHeld;
+    VT held_o[kHeld], held_g[kHeld];
+    if (live && resident) {
 #pragma unroll
-            for (int e = 0; e < V; ++e) delta = fmaf(to_f32(ov.e[e]), to_f32(gv.e[e]), delta);
+        for (int k = 0; k < kHeld; ++k) {
+            const int64_t i = (static_cast<int64_t>(k) * G + t) * V;
+            if (i < p.x_size) {
+                held_o[k] = *reinterpret_cast<const VT*>(o + i);
+                held_g[k] = *reinterpret_cast<const VT*>(g + i);
+            }
+        }
+    }
+    float delta = 0.f;
+    auto absorb = [&](const VT& ov, const VT& gv) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) delta = fmaf(to_f32(ov.e[e]), to_f32(gv.e[e]), delta);
+    };
+    if (live) {
+        if (resident) {
+#pragma unroll
+            for (int k = 0; k < kHeld; ++k)
+                if ((static_cast<int64_t>(k) * G + t) * V < p.x_size) absorb(held_o[k], held_g[k]);
+        } else {
+            for (int64_t i = static_cast<int64_t>(t) * V; i < p.x_size; i += G * V)
+                absorb(*reinterpret_cast<const VT*>(o + i), *reinterpret_cast<const VT*>(g + i));
         }
     }
     delta = wave_sum(delta);
@@ -147,13 +194,21 @@ __global__ __launch_bounds__(256) void softmax_bwd_rows_kernel(const RowParams p
         delta = (part[0] + part[1]) + (part[2] + part[3]);
     }
     if (!live) return;
-    for (int64_t i = static_cast<int64_t>(t) * V; i < p.x_size; i += G * V) {
-        const VT ov = *reinterpret_cast<const VT*>(o + i);
-        const VT gv = *reinterpret_cast<const VT*>(g + i);
+    auto emit = [&](const VT& ov, const VT& gv, int64_t i) {
         VT r;
 #pragma unroll
         for (int e = 0; e < V; ++e) r.e[e] = from_f32<T>(to_f32(ov.e[e]) * (to_f32(gv.e[e]) - delta));
         *reinterpret_cast<VT*>(gi + i) = r;
+    };
+    if (resident) {
+#pragma unroll
+        for (int k = 0; k < kHeld; ++k) {
+            const int64_t i = (static_cast<int64_t>(k) * G + t) * V;
+            if (i < p.x_size) emit(held_o[k], held_g[k], i);
+        }
+    } else {
+        for (int64_t i = static_cast<int64_t>(t) * V; i < p.x_size; i += G * V)
+            emit(*reinterpret_cast<const VT*>(o + i), *reinterpret_cast<const VT*>(g + i), i);
     }
 }
 
@@ -200,31 +255,48 @@ __global__ __launch_bounds__(256) void softmax_bwd_cols_kernel(const RowParams p
 }
 
 // ------------------------------------------------------------------ dropout
-// A thread owns 16 consecutive elements = one Philox call; BACKWARD reads grad_output instead of input.
+// A thread makes one Philox call = the 16 decisions of elements 16 t .. 16 t + 15; BACKWARD reads grad_output instead
+// of input. A wave's 1024 elements are read and written 16 bytes per lane with consecutive lanes on consecutive
+// addresses (whole cache lines per instruction), so a lane's piece belongs to another lane's Philox block: every lane
+// leaves its four words in LDS and picks up the words of its pieces from there. Blocks that are ragged or unaligned
+// fall back to a thread working through its own 16 elements.
 __device__ __forceinline__ uint32_t drop_byte(const Philox4& r, int e) { return (r.w[e >> 2] >> (8 * (e & 3))) & 0xffu; }
 
 template <typename T>
 __global__ __launch_bounds__(256) void dropout_kernel(const RowParams p, const T* __restrict__ src, T* __restrict__ dst, int64_t n) {
+    __shared__ __attribute__((aligned(16))) uint32_t words[256 * 4];
     const int64_t blk = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-    const int64_t i0 = blk * 16;
-    if (i0 >= n) return;
+    const int lane = threadIdx.x & 63;
+    uint32_t* wave_words = words + (threadIdx.x - lane) * 4;
+    const int64_t wave_i0 = (blk - lane) * 16;  // first element of this wave's 1024
     const Philox4 r = philox4x32_10(static_cast<uint32_t>(blk), static_cast<uint32_t>(blk >> 32), kDropoutStream, p.offset,
                                     p.seed_lo, p.seed_hi);
-    constexpr int V = 16 / sizeof(T);
+    *reinterpret_cast<uint4*>(wave_words + lane * 4) = uint4{r.w[0], r.w[1], r.w[2], r.w[3]};
+    __syncthreads();
+    if (wave_i0 >= n) return;
+    constexpr int V = 16 / sizeof(T);  // elements of a 16-byte piece
+    constexpr int W = V / 4;           // Philox words of a piece
+    constexpr int PPB = 16 / V;        // pieces per Philox block
     using VT = Vec<T, V>;
-    if (i0 + 16 <= n && (reinterpret_cast<uintptr_t>(src) & 15) == 0 && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+    const bool whole = wave_i0 + 1024 <= n && (reinterpret_cast<uintptr_t>(src) & 15) == 0 && (reinterpret_cast<uintptr_t>(dst) & 15) == 0;
+    if (whole) {  // (the same for every lane of the wave)
 #pragma unroll
-        for (int c = 0; c < 16 / V; ++c) {
-            const VT v = *reinterpret_cast<const VT*>(src + i0 + c * V);
+        for (int c = 0; c < PPB; ++c) {
+            const int piece = c * 64 + lane;  // of the wave's 64 PPB pieces: words piece * W .. + W - 1 of the wave
+            uint32_t w[W];
+#pragma unroll
+            for (int k = 0; k < W; ++k) w[k] = wave_words[piece * W + k];
+            const VT v = *reinterpret_cast<const VT*>(src + wave_i0 + static_cast<int64_t>(piece) * V);
             VT o;
 #pragma unroll
             for (int e = 0; e < V; ++e) {
-                const bool keep = static_cast<int>(drop_byte(r, c * V + e)) >= p.thr8;
+                const bool keep = static_cast<int>((w[e >> 2] >> (8 * (e & 3))) & 0xffu) >= p.thr8;
                 o.e[e] = from_f32<T>(keep ? to_f32(v.e[e]) * p.zscale : 0.f);
             }
-            *reinterpret_cast<VT*>(dst + i0 + c * V) = o;
+            *reinterpret_cast<VT*>(dst + wave_i0 + static_cast<int64_t>(piece) * V) = o;
         }
     } else {
+        const int64_t i0 = blk * 16;
         for (int e = 0; e < 16 && i0 + e < n; ++e) {
             const bool keep = static_cast<int>(drop_byte(r, e)) >= p.thr8;
             dst[i0 + e] = from_f32<T>(keep ? to_f32(src[i0 + e]) * p.zscale : 0.f);
