@@ -405,7 +405,7 @@ def main():
     ap.add_argument("--scenario", choices=["attention"], help="instead of the benchmark: the reference's benchmark scenario "
                     "(benchmarks/benchmarker.py --scenario attention), one JSON line")
     ap.add_argument("--mode", choices=["forward", "backward"], default="forward")
-    ap.add_argument("--dtype", choices=["float32", "float16", "bfloat16"], default="float16")
+    ap.add_argument("--dtype", choices=["float32", "float16", "bfloat16"], default="float32")
     ap.add_argument("--ceiling", action="store_true",
                     help="instead of the benchmark: print one JSON line with the MFMA ceiling of this box (random-operand "
                          "MFMA loops, a bf16 GEMM, the C3 kernels)")
