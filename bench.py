@@ -369,6 +369,12 @@ def ceiling(dev):
         tf = cus * 8 * iters * 64 * 32768.0 / ms / 1e9
         res[name] = {"ms": round(ms, 3), "tflops": round(tf, 1), "frac_of_peak": round(tf / peak, 4),
                      "busy_x_clock_GHz": round(2.4 * tf / peak, 3)}
+    ms = timed(lambda: _lib.check(lib.tri_attn_probe_mfma(3, cus, iters // 4, operands.data_ptr(), out.data_ptr(),
+                                                           torch.cuda.current_stream().cuda_stream)), 5)
+    tf = cus * 8 * (iters // 4) * 64 * 4096.0 / ms / 1e9
+    res["mfma_fp32_registers"] = {"ms": round(ms, 3), "tflops": round(tf, 1), "peak_tflops": PEAK_TFLOPS["fp32"],
+                                  "frac_of_peak": round(tf / PEAK_TFLOPS["fp32"], 4),
+                                  "busy_x_clock_GHz": round(2.4 * tf / PEAK_TFLOPS["fp32"], 3)}
     n = 8192
     a = torch.randn(n, n, device=dev).to(torch.bfloat16)
     b = torch.randn(n, n, device=dev).to(torch.bfloat16)

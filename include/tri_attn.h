@@ -196,8 +196,9 @@ int tri_attn_dropout_mask(uint64_t seed, uint64_t offset, float dropout_p, uint3
 /* Calibration helper with no counterpart in the reference: `workgroups` workgroups of 512 threads each run
  * iters x 64 bf16 32x32x16 MFMAs per wave on the caller's operand bits (operands: 16 * 512 * 16 bytes of
  * device memory read as bf16 values, e.g. random normals; out: workgroups * 512 floats).
- * mode 0: operands in registers; 1: every A operand read from LDS; 2: every LDS read feeds two MFMAs.
- * Flops per launch = workgroups * 8 * iters * 64 * 32768. Used by bench.py --ceiling. */
+ * mode 0: operands in registers; 1: every A operand read from LDS; 2: every LDS read feeds two MFMAs;
+ * 3: the fp32 instruction (v_mfma_f32_32x32x2_f32), operands in registers.
+ * Flops per launch = workgroups * 8 * iters * 64 * 32768 (mode 3: * 4096). Used by bench.py --ceiling. */
 int tri_attn_probe_mfma(int mode, int workgroups, int iters, const void* operands, float* out, void* stream);
 
 #ifdef __cplusplus

@@ -14,9 +14,10 @@ constexpr int kProbeLdsBytes = 128 * 1024;  // a wave's reads of one loop trip s
 // MODE 0: operands in registers (8 A and 8 B fragments per wave, all pairings over 8 loop trips)
 // MODE 1: every MFMA takes its A fragment from LDS (one ds_read_b128 per MFMA, as the attention kernels do)
 // MODE 2: every A fragment read from LDS feeds two MFMAs (two B fragments, two accumulators)
+// MODE 3: the fp32 instruction (v_mfma_f32_32x32x2_f32), operands in registers: 64 steps of 4096 flops per loop trip
 template <int MODE>
 __global__ __launch_bounds__(kProbeThreads) void probe_kernel(const u32x4* __restrict__ operands, float* out, int iters) {
-    __shared__ __attribute__((aligned(1024))) char smem[MODE == 0 ? 16 : kProbeLdsBytes];
+    __shared__ __attribute__((aligned(1024))) char smem[MODE == 0 || MODE == 3 ? 16 : kProbeLdsBytes];
     const int tid = threadIdx.x, lane = tid & 63;
     u32x4 a[8], b[8];
 #pragma unroll
@@ -24,7 +25,7 @@ __global__ __launch_bounds__(kProbeThreads) void probe_kernel(const u32x4* __res
         a[i] = operands[i * kProbeThreads + tid];
         b[i] = operands[(8 + i) * kProbeThreads + tid];
     }
-    if constexpr (MODE != 0) {
+    if constexpr (MODE == 1 || MODE == 2) {
         for (int i = tid; i < kProbeLdsBytes / 16; i += kProbeThreads)
             *reinterpret_cast<u32x4*>(smem + i * 16) = operands[i % (16 * kProbeThreads)];
         __syncthreads();
@@ -34,7 +35,7 @@ __global__ __launch_bounds__(kProbeThreads) void probe_kernel(const u32x4* __res
     // can be hoisted out of the loop)
     auto base_of = [&](int it) { return smem + (((it + (tid >> 6) * 8) & 63) << 10) + lane * 16; };
     u32x4 ring[8];
-    if constexpr (MODE != 0) {
+    if constexpr (MODE == 1 || MODE == 2) {
 #pragma unroll
         for (int r = 0; r < 8; ++r) ring[r] = lds_read16(base_of(0), r * 1024);
     }
@@ -44,6 +45,14 @@ __global__ __launch_bounds__(kProbeThreads) void probe_kernel(const u32x4* __res
             for (int r = 0; r < 8; ++r)
 #pragma unroll
                 for (int j = 0; j < 8; ++j) c[j & 3] = Mma<bf16_t>::run(a[j], b[(j + r) & 7], c[j & 3]);
+        } else if constexpr (MODE == 3) {
+            // (a pair of bf16 values read as one fp32 number: the upper one with some more mantissa bits)
+#pragma unroll
+            for (int r = 0; r < 8; ++r)
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    c[j & 3] = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, a[j].x),
+                                                                     __builtin_bit_cast(float, b[(j + r) & 7].x), c[j & 3], 0, 0, 0);
         } else {
             constexpr int kReads = MODE == 1 ? 64 : 32;
             const char* base = base_of(it);
@@ -75,12 +84,13 @@ using namespace tri;
 
 extern "C" int tri_attn_probe_mfma(int mode, int workgroups, int iters, const void* operands, float* out, void* stream) {
     if (operands == nullptr || out == nullptr) return TRI_ATTN_ENULL;
-    if (workgroups <= 0 || iters <= 0 || mode < 0 || mode > 2) return TRI_ATTN_ESHAPE;
+    if (workgroups <= 0 || iters <= 0 || mode < 0 || mode > 3) return TRI_ATTN_ESHAPE;
     const dim3 grid(workgroups), block(kProbeThreads);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const u32x4* ops = static_cast<const u32x4*>(operands);
     if (mode == 0) hipLaunchKernelGGL(probe_kernel<0>, grid, block, 0, st, ops, out, iters);
     else if (mode == 1) hipLaunchKernelGGL(probe_kernel<1>, grid, block, 0, st, ops, out, iters);
-    else hipLaunchKernelGGL(probe_kernel<2>, grid, block, 0, st, ops, out, iters);
+    else if (mode == 2) hipLaunchKernelGGL(probe_kernel<2>, grid, block, 0, st, ops, out, iters);
+    else hipLaunchKernelGGL(probe_kernel<3>, grid, block, 0, st, ops, out, iters);
     return static_cast<int>(hipGetLastError());
 }
