@@ -298,12 +298,22 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void mfma32_dq_kernel(const 
                 s = mma32(kf.w, qf[4 * j + 3], s);
                 dp = mma32(vf.w, gf[4 * j + 3], dp);
             }
-            float ds[16];
+            // (one branch per tile decides about the mask: a branch per element costs more than the arithmetic it guards)
+            float ds[16], mk[16];
+            if (p.mask) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int key = k0 + c_row(i, h);
+                    mk[i] = key < p.S ? load_mask_elem(p.mask, p.mask_dtype, mrow + key) * kLog2e : 0.f;
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) mk[i] = 0.f;
+            }
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int key = k0 + c_row(i, h);
-                float v = s[i] * p.scale_log2;
-                if (p.mask && key < p.S) v = fmaf(load_mask_elem(p.mask, p.mask_dtype, mrow + key), kLog2e, v);
+                const float v = fmaf(s[i], p.scale_log2, mk[i]);
                 const bool visible = key < p.S && (!p.causal || key <= qrow);
                 ds[i] = visible ? fast_exp2(v - lse) : 0.f;
             }
@@ -452,15 +462,23 @@ __global__ __launch_bounds__(256, D >= 64 ? 1 : 2) void mfma32_dkdv_kernel(const
                 dp = mma32(ga.z, vf[4 * j + 2], dp);
                 s = mma32(qa.w, kf[4 * j + 3], s);
                 dp = mma32(ga.w, vf[4 * j + 3], dp);
-                __builtin_amdgcn_sched_barrier(0);
             }
             // this lane: its key, rows r0 + c_row(i, h)
-            float pr[16], ds[16];
+            float pr[16], ds[16], mk[16];
+            if (p.mask) {  // (one branch per tile, not one per element)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int row = r0 + c_row(i, h);
+                    mk[i] = row < p.S ? load_mask_elem(p.mask, p.mask_dtype, mcol + row * p.ms[2]) * kLog2e : 0.f;
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) mk[i] = 0.f;
+            }
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int row = r0 + c_row(i, h);
-                float v = s[i] * p.scale_log2;
-                if (p.mask && row < p.S) v = fmaf(load_mask_elem(p.mask, p.mask_dtype, mcol + row * p.ms[2]), kLog2e, v);
+                const float v = fmaf(s[i], p.scale_log2, mk[i]);
                 const bool visible = row < p.S && key_ok && (!p.causal || key <= row);
                 pr[i] = visible ? fast_exp2(v - sLse[c_row(i, h)]) : 0.f;
             }
@@ -491,7 +509,6 @@ __global__ __launch_bounds__(256, D >= 64 ? 1 : 2) void mfma32_dkdv_kernel(const
                     dv[db] = mma32(in ? grow[32 * db] : 0.f, pr[r], dv[db]);
                     dk[db] = mma32(in ? qrow[32 * db] : 0.f, ds[r], dk[db]);
                 }
-                __builtin_amdgcn_sched_barrier(0);  // (operand reads stay next to their use: registers are short)
             }
         }
         __syncthreads();
@@ -621,14 +638,22 @@ __global__ __launch_bounds__(256, 1) void mfma32_dkdv_split_kernel(const KParams
                 dp = mma32(ga.z, vf.z, dp);
                 s = mma32(qa.w, kf.w, s);
                 dp = mma32(ga.w, vf.w, dp);
-                __builtin_amdgcn_sched_barrier(0);
             }
-            float pr[16], ds[16];
+            float pr[16], ds[16], mk[16];
+            if (p.mask) {  // (one branch per tile, not one per element)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int row = r0 + c_row(i, h);
+                    mk[i] = row < p.S ? load_mask_elem(p.mask, p.mask_dtype, mcol + row * p.ms[2]) * kLog2e : 0.f;
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) mk[i] = 0.f;
+            }
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int row = r0 + c_row(i, h);
-                float v = s[i] * p.scale_log2;
-                if (p.mask && row < p.S) v = fmaf(load_mask_elem(p.mask, p.mask_dtype, mcol + row * p.ms[2]), kLog2e, v);
+                const float v = fmaf(s[i], p.scale_log2, mk[i]);
                 const bool visible = row < p.S && key_ok && (!p.causal || key <= row);
                 pr[i] = visible ? fast_exp2(v - sLse[kTile32 * rh + c_row(i, h)]) : 0.f;
             }
@@ -657,7 +682,6 @@ __global__ __launch_bounds__(256, 1) void mfma32_dkdv_split_kernel(const KParams
                     dv[db] = mma32(grow[32 * db], pr[r], dv[db]);
                     dk[db] = mma32(qrow[32 * db], ds[r], dk[db]);
                 }
-                __builtin_amdgcn_sched_barrier(0);
             }
         }
         __syncthreads();
