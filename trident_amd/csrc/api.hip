@@ -43,7 +43,6 @@ int make_params(const TriAttnArgs* a, int need, KParams* p) {
     }
     memset(p, 0, sizeof(*p));
     int rc;
-    { static const int xf = getenv("TRI_X") ? atoi(getenv("TRI_X")) : 0; p->xflag = xf; }  // TEMP
     if (need & 1) {
         if (!a->q || !a->k || !a->v || !a->o || !a->lse) return TRI_ATTN_ENULL;
         if ((rc = check_strides(a->q_stride)) || (rc = check_strides(a->k_stride)) ||

@@ -36,7 +36,6 @@ struct KParams {
     float scale;       // softmax_scale
     float scale_log2;  // softmax_scale * log2(e)
     uint32_t seed_lo, seed_hi, offset;
-    int xflag;  // TEMP experiment switch
     int dmask_acc;     // dmask is summed over a broadcast dimension (stride 0): fp32 buffer, atomic adds
     int thr8;          // 0 = no dropout; keep iff u8 >= thr8
     float zscale;      // 256 / (256 - thr8), 0 when thr8 == 256
