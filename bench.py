@@ -375,6 +375,18 @@ def ceiling(dev):
     res["mfma_fp32_registers"] = {"ms": round(ms, 3), "tflops": round(tf, 1), "peak_tflops": PEAK_TFLOPS["fp32"],
                                   "frac_of_peak": round(tf / PEAK_TFLOPS["fp32"], 4),
                                   "busy_x_clock_GHz": round(2.4 * tf / PEAK_TFLOPS["fp32"], 3)}
+    # vector work of one wave beside another wave's MFMAs on the same SIMD: alone, alone, together (ms)
+    co = {}
+    for matrix, mname in ((0, "bf16_32x32x16"), (1, "fp32_32x32x2")):
+        for valu, vname in ((0, "fma"), (1, "exp2"), (2, "fma_max_exp2")):
+            row = {}
+            for who, wname in ((1, "matrix_ms"), (2, "vector_ms"), (3, "both_ms")):
+                row[wname] = round(timed(lambda: _lib.check(lib.tri_attn_probe_coexec(
+                    matrix, valu, who, cus, 2000, operands.data_ptr(), out.data_ptr(),
+                    torch.cuda.current_stream().cuda_stream)), 3), 3)
+            row["hidden_fraction_of_vector_work"] = round((row["matrix_ms"] + row["vector_ms"] - row["both_ms"]) / row["vector_ms"], 3)
+            co[mname + "+" + vname] = row
+    res["coexecution"] = co
     n = 8192
     a = torch.randn(n, n, device=dev).to(torch.bfloat16)
     b = torch.randn(n, n, device=dev).to(torch.bfloat16)
@@ -390,6 +402,18 @@ def ceiling(dev):
                              "executed_tflops": round(executed[k] * unit / v / 1e9, 1),
                              "executed_frac_of_peak": round(executed[k] * unit / v / 1e9 / peak, 4)}
                         for k, v in pk.items() if k in executed}
+    # If vector work beside MFMAs costs its full time (coexecution above: hidden fraction about 0 under sustained load), a
+    # kernel cannot be faster than its MFMAs at the LDS-fed rate plus its per-score vector work (one fma, max, exp2 mix per
+    # score, the probe's rate: 256 lanes x 32 values x 2000 trips per CU in vector_ms).
+    w = pth.w
+    scores = w.B * w.H * w.S * w.S * (0.5 if w.is_causal else 1.0)
+    mix = co["bf16_32x32x16+fma_max_exp2"]
+    vec_ms = scores * mix["vector_ms"] / (cus * 256 * 32 * 2000.0)
+    for k in res["c3_kernels"]:
+        mfma_ms = executed[k] * unit / (res["mfma_lds_1_read_per_mfma"]["tflops"] * 1e9)
+        row = res["c3_kernels"][k]
+        row["additive_floor_ms"] = round(mfma_ms + vec_ms, 4)
+        row["floor_over_measured"] = round((mfma_ms + vec_ms) / row["ms"], 3)
     return res
 
 

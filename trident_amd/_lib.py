@@ -100,6 +100,7 @@ EXPORTS = (
     "tri_attn_classify_mask",
     "tri_attn_mask_classes_size",
     "tri_attn_probe_mfma",
+    "tri_attn_probe_coexec",
 )
 
 _lib = None
@@ -142,6 +143,9 @@ def lib():
         cdll.tri_attn_probe_mfma.restype = ctypes.c_int
         cdll.tri_attn_probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
                                              ctypes.c_void_p, ctypes.c_void_p]
+        cdll.tri_attn_probe_coexec.restype = ctypes.c_int
+        cdll.tri_attn_probe_coexec.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                               ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
         if cdll.tri_attn_version() != ABI_VERSION:
             raise RuntimeError("libtrident_attn.so ABI version mismatch: rebuild it")
         _lib = cdll
