@@ -48,7 +48,7 @@ BASELINE_KERNELS = {
     "mfma_fwd_kernel<__bf16, 128, 8, true, 0, true, false>": "C5 fwd",
     "mfma_dq_phased_kernel<__bf16, 128, true, true, true>": "C5 dQ + delta",
     "mfma_dkdv_phased_kernel<__bf16, 128, true, true>": "C5 dK/dV",
-    "generic_fwd_kernel<float, 32>": "C1 fwd",
+    "mfma32_fwd_kernel<float, 32>": "C1 fwd",
 }
 _FIELDS = [("TotalSGPRs", "sgpr"), ("VGPRs", "vgpr"), ("AGPRs", "agpr"), ("ScratchSize [bytes/lane]", "scratch"),
            ("Occupancy [waves/SIMD]", "occupancy"), ("SGPRs Spill", "sgpr_spill"), ("VGPRs Spill", "vgpr_spill"),
