@@ -1322,7 +1322,6 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
     const int n_blocks = (p.S - row_first) / kBR;   // >= 4, even
     const uint32_t qoff = static_cast<uint32_t>(Tile::src_off(wave, lane, qrow_bytes));
     const uint32_t goff = static_cast<uint32_t>(Tile::src_off(wave, lane, grow_bytes));
-    auto slot_of = [&](int r) { return smem + ((r + kSlots) % kSlots) * kSlotBytes; };
     // Blocks are requested in order, one per phase (block ph + 4 in phase ph) after the first four: the
     // source pointers and the ring slot advance with every call. Even waves fetch the 32 lse values of a
     // block, odd waves its 32 delta values (lanes 32-63 repeat them).
@@ -1409,25 +1408,32 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
 
     // whether this pair has anything in block r (under the causal mask: rows at or below its first key)
     auto block_on = [&](int r) { return r >= 0 && r < n_blocks && (!CAUSAL || r >= kb); };
-    auto clamp_block = [&](int r) { return r < 0 ? 0 : (r >= n_blocks ? n_blocks - 1 : r); };
 
     constexpr float kFoldUnit = 256.f;  // the constant the split terms multiply (keeps f16 terms in range)
     const float neg_inv_c = -1.f / c;
     f32x16 sc_s, sc_dp;  // S - lse / c and dP - delta of this member's next block
     u32x4 ring[kRing];
-    // fragment n of a matrix phase that adds blocks ra and rb and scores block rs
-    auto frag = [&](int ra, int rb, int rs, int n) {
+    // Ring slots are named by their byte offset in LDS and stepped from block to block (a slot index taken modulo 7
+    // for every block a phase touches costs a dozen scalar instructions each time).
+    constexpr int kRingBytes = kSlots * kSlotBytes;
+    auto slot_step = [&](int so, int d) {
+        int t = so + d * kSlotBytes;
+        t = t >= kRingBytes ? t - kRingBytes : t;
+        return t < 0 ? t + kRingBytes : t;
+    };
+    // fragment n of a matrix phase that adds the blocks in slots sa and sb and scores the block in slot ss
+    auto frag = [&](int sa, int sb, int ss, int n) {
         if (n < 2 * kAccSteps) {
-            const char* slot = slot_of(n < kAccSteps ? ra : rb);
+            const char* slot = smem + (n < kAccSteps ? sa : sb);
             const int m = n % kAccSteps;
             const int d = m % DH, which = (m / DH) % 2, g = m / (2 * DH);
             const int db = DH * member + d;
             return Tile::tr_frag(slot + (which ? 0 : kHalfBytes), tr_off0 ^ (db << 6), tr_off1 ^ (db << 6), g);
         }
         const int m = n - 2 * kAccSteps;
-        return lds_read16(slot_of(rs) + (m < KK ? 0 : kHalfBytes), row_off0 ^ ((m % KK) << 5));
+        return lds_read16(smem + ss + (m < KK ? 0 : kHalfBytes), row_off0 ^ ((m % KK) << 5));
     };
-    auto matrix_phase = [&](auto with_acc, int ra, int rb, int rs, bool own_on = true, bool score_on = true) {
+    auto matrix_phase = [&](auto with_acc, int sa, int sb, int ss, bool own_on = true, bool score_on = true) {
         constexpr int first = decltype(with_acc)::value ? 0 : 2 * kAccSteps;
         f32x16 s = zero16(), dp = zero16();
         // One more MFMA each puts -lse / c and -delta under S and dP (a row's value split into three 16-bit
@@ -1439,7 +1445,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
             const int slot = (n - first) % kRing;
             if ((n == kAccSteps && !own_on && !score_on) || (n == 2 * kAccSteps && !score_on)) break;
             if (n == first) {
-                const float* sLse = reinterpret_cast<const float*>(slot_of(rs) + 2 * kHalfBytes);
+                const float* sLse = reinterpret_cast<const float*>(smem + ss + 2 * kHalfBytes);
                 row_lse = sLse[l32];
                 if constexpr (!DROPOUT) row_delta = sLse[64 + l32];
             }
@@ -1463,7 +1469,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
                 if (m < KK) s = Mma<T>::run(ring[slot], kf[m], s);
                 else dp = Mma<T>::run(ring[slot], vf[m - KK], dp);
             }
-            if (n + kRing < kSteps) ring[slot] = frag(ra, rb, rs, n + kRing);
+            if (n + kRing < kSteps) ring[slot] = frag(sa, sb, ss, n + kRing);
             __builtin_amdgcn_sched_barrier(0);
         }
         sc_s = s;
@@ -1474,7 +1480,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
 
     // P = exp2(c S') and dS = P dP' of the block whose first row is rb, eight rows at a time, packed as soon as
     // they are done; only the block on the diagonal pays for the causal comparison (scores above it become -inf)
-    auto softmax_backward = [&](bool on_diagonal, int rb, int r) {
+    auto softmax_backward = [&](bool on_diagonal, int rb, int so) {
         if (on_diagonal) {
             // a real branch, taken for one block per workgroup; the row base goes through a scalar register the
             // compiler cannot see through, so that the 16 comparisons are made here and not kept as lane masks
@@ -1485,7 +1491,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
             for (int i = 0; i < 16; ++i) sc_s[i] = key <= rbo + c_row(i, h) ? sc_s[i] : -INFINITY;
         }
         const f32x16 s = sc_s, dp = sc_dp;
-        const float* sDelta = reinterpret_cast<const float*>(slot_of(r) + 2 * kHalfBytes) + 64;
+        const float* sDelta = reinterpret_cast<const float*>(smem + so + 2 * kHalfBytes) + 64;
         Philox4 mine;  // the block of rows rb + 8 (lane % 4) + 4 h .. +3: this lane's share of the quad's four
         if constexpr (DROPOUT) mine = dropout_block(p, bh, (rb + 8 * (lane & 3) + 4 * h) >> 2, key >> 2);
 #pragma unroll
@@ -1522,10 +1528,10 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
         }
     };
     // vector phase for block r (this member's): P and dS from sc_s, sc_dp
-    auto vector_phase = [&](int r) {
+    auto vector_phase = [&](int r, int so) {
         if (block_on(r)) {
             const int rb = row_first + r * kBR;
-            softmax_backward(CAUSAL && r == kb, rb, r);
+            softmax_backward(CAUSAL && r == kb, rb, so);
         } else {
 #pragma unroll
             for (int g = 0; g < 2; ++g) cur_p[g] = cur_s[g] = u32x4{0, 0, 0, 0};
@@ -1533,7 +1539,9 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
     };
     // the second half of a vector phase in global phase ph, for a member whose block is r: publish, fetch
     // the partner's block r-1, request the first fragments of the matrix phase, meet the barrier
-    auto close_vector_phase = [&](int ph, int r) {
+    // (so: the slot of block r; block r - 1 sits one slot before it, block r + 2 two after; at the ends of the range the
+    // neighbour that does not exist is replaced by one that does, its P and dS are zero)
+    auto close_vector_phase = [&](int ph, int r, int so) {
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
             *reinterpret_cast<u32x4*>(my_xch + g * 1024) = cur_p[g];
@@ -1546,9 +1554,10 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
             par_p[g] = *reinterpret_cast<const u32x4*>(peer_xch + g * 1024);
             par_s[g] = *reinterpret_cast<const u32x4*>(peer_xch + (2 + g) * 1024);
         }
-        const int ra = clamp_block(r - 1), rb = clamp_block(r);
+        const int before = slot_step(so, -1);
+        const int sa = r > 0 ? before : so, sb = r < n_blocks ? so : before;
 #pragma unroll
-        for (int n = 0; n < kRing; ++n) ring[n] = frag(ra, rb, r + 2, n);
+        for (int n = 0; n < kRing; ++n) ring[n] = frag(sa, sb, slot_step(so, 2), n);
         // LDS operations of a wave complete in order: once at most the 4 + 2 kRing reads above are
         // outstanding, the slot is published
         static_assert(4 + 2 * kRing <= 15, "lgkmcnt range");
@@ -1559,7 +1568,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
         asm volatile("s_barrier" ::: "memory");  // (the reads above stay in flight)
         __builtin_amdgcn_sched_barrier(0);
     };
-    auto run_matrix_phase = [&](int ph, int r) {
+    auto run_matrix_phase = [&](int ph, int r, int so) {
         // this phase's loads first, while the ring's first fragments are still on their way (after the MFMAs
         // they cost 1-1.6 % more cycles, between them 23 %)
         // (the last rounds have no own block to add and no block r + 2 to score: those steps are left out, except
@@ -1567,7 +1576,9 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
         issue_block();
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_setprio(2);
-        matrix_phase(Yes{}, clamp_block(r - 1), clamp_block(r), r + 2, DROPOUT || r < n_blocks, DROPOUT || r + 2 < n_blocks);
+        const int before = slot_step(so, -1);
+        matrix_phase(Yes{}, r > 0 ? before : so, r < n_blocks ? so : before, slot_step(so, 2), DROPOUT || r < n_blocks,
+                     DROPOUT || r + 2 < n_blocks);
         __builtin_amdgcn_s_setprio(0);
         wait_blocks(ph);
         __builtin_amdgcn_sched_barrier(0);
@@ -1583,30 +1594,34 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
     // before phase 0: S and dP of each member's first block (member 0: block 0, member 1: block 1)
     {
 #pragma unroll
-        for (int n = 0; n < kRing; ++n) ring[n] = frag(0, 0, member, 2 * kAccSteps + n);
+        for (int n = 0; n < kRing; ++n) ring[n] = frag(0, 0, member * kSlotBytes, 2 * kAccSteps + n);
         __builtin_amdgcn_sched_barrier(0);
-        matrix_phase(No{}, 0, 0, member);
+        matrix_phase(No{}, 0, 0, member * kSlotBytes);
         lds_barrier();
     }
     const int n_iter = n_blocks / 2;
     if (member == 0) {
         refresh_lane_offsets();
+        int so = 0;  // slot of block r
 #pragma unroll 1
         for (int t = 0; t <= n_iter; ++t) {   // the last round only adds member 1's last block
             const int r = 2 * t;
-            vector_phase(r);
-            close_vector_phase(2 * t, r);
-            run_matrix_phase(2 * t + 1, r);
+            vector_phase(r, so);
+            close_vector_phase(2 * t, r, so);
+            run_matrix_phase(2 * t + 1, r, so);
+            so = slot_step(so, 2);
         }
     } else {
         refresh_lane_offsets();
         idle_phase(0);
+        int so = kSlotBytes;  // slot of block r
 #pragma unroll 1
         for (int t = 0; t < n_iter; ++t) {
             const int r = 2 * t + 1;
-            vector_phase(r);
-            close_vector_phase(2 * t + 1, r);
-            run_matrix_phase(2 * t + 2, r);
+            vector_phase(r, so);
+            close_vector_phase(2 * t + 1, r, so);
+            run_matrix_phase(2 * t + 2, r, so);
+            so = slot_step(so, 2);
         }
         idle_phase(2 * n_iter + 1);
     }
