@@ -461,6 +461,27 @@ def test_views_that_are_not_four_element_aligned_take_the_vector_alu_kernels(dty
     parity.close(dv, dv_r, dtype, "odd view dV", a_dv)
 
 
+def _random_cases(count, seed):
+    rng = np.random.RandomState(seed)
+    cases = []
+    for i in range(count):
+        dtype = [torch.float32, torch.bfloat16, torch.float16][rng.randint(3)]
+        D = [16, 32, 64, 128][rng.randint(4)]
+        S = int(rng.choice([rng.randint(1, 40), rng.randint(40, 300), rng.randint(300, 700), 128 * rng.randint(1, 6)]))
+        variant = ["plain", "causal", "mask", "mask16", "dropout", "causal+dropout"][rng.randint(6)]
+        if variant == "mask16" and dtype == torch.float32:
+            variant = "mask"
+        cases.append((dtype, S, D, variant, int(rng.randint(1, 3)), int(rng.randint(1, 4)), 9000 + i))
+    return cases
+
+
+@pytest.mark.parametrize("dtype,S,D,variant,batches,heads,seed", _random_cases(48, 20240611))
+def test_random_problems(dtype, S, D, variant, batches, heads, seed, device):
+    """A fixed pseudo-random sample of (dtype, length, head size, mask mode, dropout, batch, heads): whatever kernel
+    family the dispatch picks, forward, LSE, delta and the three gradients match the oracle."""
+    _abi_case(device, dtype, S, D, variant, seed, batches=batches, heads=heads)
+
+
 # ------------------------------------------------------------------ tile counts of the phased kernels
 @pytest.mark.parametrize("variant", ["plain", "causal", "causal+dropout"])
 @pytest.mark.parametrize("S,D", [(256, 128), (768, 128), (1280, 128), (768, 64), (1024, 64)])
