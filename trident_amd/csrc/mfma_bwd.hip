@@ -53,11 +53,12 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
     constexpr int DB = D / 32;
     constexpr int kBlocksPerWave = 2 * Tile::kBlocks / NW;  // LDS-direct loads per wave and tile
     static_assert(2 * Tile::kBlocks % NW == 0, "tile blocks must divide among the waves");
-    // An fp32 mask block of a wave (32 rows x 64 keys) goes through a private 8 KiB LDS region when
-    // it fits (D = 64): lanes own rows, so direct loads would touch 32 cache lines per instruction,
-    // while LDS-direct loads fetch whole 256-byte rows. Geometry of a 32-row SwzTile<128>.
-    constexpr bool kMaskViaLds = MASK == kMaskF32 && D == 64;
-    using MaskTile = SwzTile<128>;
+    // A mask block of a wave (32 rows x 64 keys) goes through a private LDS region (8 KiB fp32, 4 KiB for a mask of
+    // the operand type) when it fits (D = 64): lanes own rows, so direct loads would touch 32 cache lines per
+    // instruction, while LDS-direct loads fetch whole rows. Geometry of a 32-row SwzTile<128> / SwzTile<64>.
+    constexpr bool kMaskViaLds = MASK != kNoMask && D == 64;
+    constexpr int kMaskElt = MASK == kMaskF32 ? 4 : 2;
+    using MaskTile = std::conditional_t<MASK == kMaskF32, SwzTile<128>, SwzTile<64>>;
     constexpr int kMaskBytes = 32 * MaskTile::kRowBytes;
     constexpr int kMaskLoads = kMaskBytes / 1024;
     __shared__ __attribute__((aligned(1024))) char smem[kStages * kStageBytes + (kMaskViaLds ? NW * kMaskBytes : 0)];
@@ -137,12 +138,12 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
         if constexpr (kMaskViaLds) {
             if (mask_is_zero(t)) return;
             const char* src = static_cast<const char*>(p.mask) +
-                              (b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(wrow0) * p.ms[2] + t * kBN) * 4;
+                              (b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(wrow0) * p.ms[2] + t * kBN) * kMaskElt;
             int l = lane;
             asm volatile("" : "+v"(l));  // offsets recomputed per tile rather than kept in registers
 #pragma unroll
             for (int blk = 0; blk < kMaskLoads; ++blk)
-                lds_direct_load16(src, static_cast<uint32_t>(MaskTile::src_off(blk, l, p.ms[2] * 4)), mask_lds + blk * 1024);
+                lds_direct_load16(src, static_cast<uint32_t>(MaskTile::src_off(blk, l, p.ms[2] * kMaskElt)), mask_lds + blk * 1024);
         }
     };
     // issue order: mask 0, tiles 0 1 2, then per tile j: mask j+1, tile j+3
@@ -183,9 +184,15 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
                 for (int i = 0; i < 32; ++i) mk2[i] = 0.f;
             } else {
 #pragma unroll
-                for (int g = 0; g < 8; ++g) {
-                    const f32x4 v = *reinterpret_cast<const f32x4*>(mask_lds + MaskTile::off(l32, 2 * g + h));
-                    mk2[4 * g + 0] = v.x; mk2[4 * g + 1] = v.y; mk2[4 * g + 2] = v.z; mk2[4 * g + 3] = v.w;
+                for (int g = 0; g < 8; ++g) {  // keys 8 g + 4 h .. + 3 of this lane's row
+                    if constexpr (MASK == kMaskF32) {
+                        const f32x4 v = *reinterpret_cast<const f32x4*>(mask_lds + MaskTile::off(l32, 2 * g + h));
+                        mk2[4 * g + 0] = v.x; mk2[4 * g + 1] = v.y; mk2[4 * g + 2] = v.z; mk2[4 * g + 3] = v.w;
+                    } else {
+                        const u32x2 v = *reinterpret_cast<const u32x2*>(mask_lds + MaskTile::off(l32, g) + 8 * h);
+                        mk2[4 * g + 0] = Mma<T>::lo(v.x); mk2[4 * g + 1] = Mma<T>::hi(v.x);
+                        mk2[4 * g + 2] = Mma<T>::lo(v.y); mk2[4 * g + 3] = Mma<T>::hi(v.y);
+                    }
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // region read before it is refilled
             }
@@ -594,12 +601,13 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
     constexpr int kBlocksPerWave = 2 * Tile::kBlocks / NW;
     constexpr int kLoadsPerTile = kBlocksPerWave + 1;            // + lse or delta: exact for every wave
     static_assert(2 * Tile::kBlocks % NW == 0, "tile blocks must divide among the waves");
-    // An fp32 mask block of a wave (64 rows x its 32 keys) goes through a private 8 KiB LDS region when
-    // it fits (D = 64). Plain loads would be tracked by the compiler, whose waits for them also drain
-    // the LDS-direct tile loads issued in between (the counter completes in order), which makes the
-    // tile prefetch synchronous. Geometry of a 64-row SwzTile<64> (128-byte rows = 32 keys).
-    constexpr bool kMaskViaLds = MASK == kMaskF32 && D == 64;
-    using MaskTile = SwzTile<64>;
+    // A mask block of a wave (64 rows x its 32 keys) goes through a private LDS region (8 KiB fp32, 4 KiB for a mask
+    // of the operand type) when it fits (D = 64). Plain loads would be tracked by the compiler, whose waits for them
+    // also drain the LDS-direct tile loads issued in between (the counter completes in order), which makes the
+    // tile prefetch synchronous. Geometry of a 64-row SwzTile<64> / SwzTile<32> (128- or 64-byte rows = 32 keys).
+    constexpr bool kMaskViaLds = MASK != kNoMask && D == 64;
+    constexpr int kMaskElt = MASK == kMaskF32 ? 4 : 2;
+    using MaskTile = std::conditional_t<MASK == kMaskF32, SwzTile<64>, SwzTile<32>>;
     constexpr int kMaskLoads = MaskTile::kBlocks;
     __shared__ __attribute__((aligned(1024))) char smem[kStages * kStageBytes + (kMaskViaLds ? NW * MaskTile::kBytes : 0)];
 
@@ -692,12 +700,12 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
         if constexpr (kMaskViaLds) {
             if (mask_is_zero(t)) return;
             const char* src = static_cast<const char*>(p.mask) +
-                              (b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(t) * kBN * p.ms[2] + wkey0) * 4;
+                              (b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(t) * kBN * p.ms[2] + wkey0) * kMaskElt;
             int l = lane;
             asm volatile("" : "+v"(l));  // offsets recomputed per tile rather than kept in registers
 #pragma unroll
             for (int blk = 0; blk < kMaskLoads; ++blk)
-                lds_direct_load16(src, static_cast<uint32_t>(MaskTile::src_off(blk, l, p.ms[2] * 4)), mask_lds + blk * 1024);
+                lds_direct_load16(src, static_cast<uint32_t>(MaskTile::src_off(blk, l, p.ms[2] * kMaskElt)), mask_lds + blk * 1024);
         }
     };
     // issue order: mask block of the first tile, three tiles, then per tile j: mask j+1, tile j+3
@@ -736,8 +744,13 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
                 for (int i = 0; i < 32; ++i) mk2[i] = 0.f;
             } else {
 #pragma unroll
-                for (int i = 0; i < 32; ++i)
-                    mk2[i] = *reinterpret_cast<const float*>(mask_lds + MaskTile::off(32 * (i >> 4) + c_row(i & 15, h), l32 >> 2) + (l32 & 3) * 4);
+                for (int i = 0; i < 32; ++i) {  // row 32 (i / 16) + c_row(i % 16, h), this lane's key
+                    const int row = 32 * (i >> 4) + c_row(i & 15, h);
+                    if constexpr (MASK == kMaskF32)
+                        mk2[i] = *reinterpret_cast<const float*>(mask_lds + MaskTile::off(row, l32 >> 2) + (l32 & 3) * 4);
+                    else
+                        mk2[i] = to_f32(*reinterpret_cast<const T*>(mask_lds + MaskTile::off(row, l32 >> 3) + (l32 & 7) * 2));
+                }
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // region read before it is refilled
             }
             if (j + 1 < n_tiles) issue_mask(j + 1);

@@ -48,12 +48,13 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     constexpr int kSteps = 2 * KK;    // MFMAs of S^T per tile
     constexpr int kPvSteps = 4 * DB;  // MFMAs of O^T per tile
     constexpr int kRing = 6;          // operand fragments in flight
-    // An fp32 mask block of a wave (32 rows x 64 keys) goes through a private 8 KiB LDS region when
-    // it fits (D = 64): lanes own rows, so direct loads would touch 32 cache lines per instruction,
-    // while LDS-direct loads fetch whole 256-byte rows and the swizzled tile is read back without
-    // bank conflicts. The region has the geometry of a 32-row SwzTile<128> (256-byte rows).
-    constexpr bool kMaskViaLds = MASK == kMaskF32 && D == 64;
-    using MaskTile = SwzTile<128>;
+    // A mask block of a wave (32 rows x 64 keys) goes through a private LDS region (8 KiB for an fp32 mask, 4 KiB
+    // for one of the operand type) when it fits (D = 64): lanes own rows, so direct loads would touch 32 cache
+    // lines per instruction, while LDS-direct loads fetch whole rows (256 or 128 bytes) and the swizzled tile is
+    // read back 16 or 8 bytes at a time. The region has the geometry of a 32-row SwzTile<128> / SwzTile<64>.
+    constexpr bool kMaskViaLds = MASK != kNoMask && D == 64;
+    constexpr int kMaskElt = MASK == kMaskF32 ? 4 : 2;
+    using MaskTile = std::conditional_t<MASK == kMaskF32, SwzTile<128>, SwzTile<64>>;
     constexpr int kMaskBytes = 32 * MaskTile::kRowBytes;
     // Without an additive mask the 8-wave kernel is persistent: one workgroup per CU walks several (head, row
     // tile) items, and requests the Q rows and the first tiles of its next item before it stores the current
@@ -123,12 +124,12 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
         if constexpr (kMaskViaLds) {
             if (mask_is_zero(t)) return;
             const char* src = static_cast<const char*>(p.mask) +
-                              (b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(wrow0) * p.ms[2] + t * kBN) * 4;
+                              (b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(wrow0) * p.ms[2] + t * kBN) * kMaskElt;
             int l = lane;
             asm volatile("" : "+v"(l));  // offsets recomputed per tile rather than kept in registers
 #pragma unroll
             for (int blk = 0; blk < kMaskBytes / 1024; ++blk)
-                lds_direct_load16(src, static_cast<uint32_t>(MaskTile::src_off(blk, l, p.ms[2] * 4)), mask_lds + blk * 1024);
+                lds_direct_load16(src, static_cast<uint32_t>(MaskTile::src_off(blk, l, p.ms[2] * kMaskElt)), mask_lds + blk * 1024);
         }
     };
     issue_mask(0);
@@ -238,9 +239,15 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
             } else {
                 if (!first) wait_loads(false, tile_in_flight);
 #pragma unroll
-                for (int g = 0; g < 8; ++g) {
-                    const f32x4 v = *reinterpret_cast<const f32x4*>(mask_lds + MaskTile::off(l32, 8 * (g >> 2) + 2 * (g & 3) + h));
-                    mk[4 * g + 0] = v.x; mk[4 * g + 1] = v.y; mk[4 * g + 2] = v.z; mk[4 * g + 3] = v.w;
+                for (int g = 0; g < 8; ++g) {  // keys 32 (g / 4) + 8 (g % 4) + 4 h .. + 3 of this lane's row
+                    if constexpr (MASK == kMaskF32) {
+                        const f32x4 v = *reinterpret_cast<const f32x4*>(mask_lds + MaskTile::off(l32, 8 * (g >> 2) + 2 * (g & 3) + h));
+                        mk[4 * g + 0] = v.x; mk[4 * g + 1] = v.y; mk[4 * g + 2] = v.z; mk[4 * g + 3] = v.w;
+                    } else {
+                        const u32x2 v = *reinterpret_cast<const u32x2*>(mask_lds + MaskTile::off(l32, 4 * (g >> 2) + (g & 3)) + 8 * h);
+                        mk[4 * g + 0] = Mma<T>::lo(v.x); mk[4 * g + 1] = Mma<T>::hi(v.x);
+                        mk[4 * g + 2] = Mma<T>::lo(v.y); mk[4 * g + 3] = Mma<T>::hi(v.y);
+                    }
                 }
             }
             // the values are in registers: the region can take the next block

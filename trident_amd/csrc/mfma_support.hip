@@ -113,7 +113,9 @@ bool mfma_supported(int which, int dtype, const KParams& p) {
     if (p.mask != nullptr) {
         if (p.mask_dtype != TRI_ATTN_F32 && p.mask_dtype != dtype) return false;
         if (!aligned16(p.mask)) return false;
-        if ((p.ms[0] % 4) || (p.ms[1] % 4) || (p.ms[2] % 4)) return false;
+        // mask rows are fetched 16 bytes at a time (D = 64, through LDS) or 8 / 16 bytes at a time (D = 128)
+        const int64_t quantum = p.mask_dtype == TRI_ATTN_F32 ? 4 : 8;
+        if ((p.ms[0] % quantum) || (p.ms[1] % quantum) || (p.ms[2] % quantum)) return false;
         if (p.ms[2] < 0 || p.ms[2] >= (int64_t{1} << 24)) return false;  // 32-bit offsets inside a mask block
     }
     switch (which) {
