@@ -466,7 +466,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
 #pragma unroll
                         for (int bb = 0; bb < 4; ++bb) {
                             const bool keep = static_cast<int>((w[g] >> (8 * bb)) & 0xffu) >= p.thr8;
-                            x[16 * kb + 4 * g + bb] = keep ? x[16 * kb + 4 * g + bb] * p.zscale : 0.f;
+                            x[16 * kb + 4 * g + bb] = keep ? x[16 * kb + 4 * g + bb] : 0.f;  // (the 1 / (1 - p) factor: at the end)
                         }
                 }
             }
@@ -516,7 +516,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     if (kPingPong && group == 0) lds_barrier();  // group 1 is still in its last matrix phase
 
     l = DROPOUT ? sum_xor32(l) : lacc[0];
-    const float inv = 1.f / l;
+    const float inv = (DROPOUT ? p.zscale : 1.f) / l;
     // every wave is out of the loop: the ring is free (for the waves' private transposition patches, and for
     // the first tiles of the next item)
     lds_barrier();
