@@ -197,3 +197,16 @@ def test_product_does_not_import_oracle():
             if name.endswith((".py", ".hip", ".hpp", ".h")):
                 text = open(os.path.join(dirpath, name)).read()
                 assert "oracle" not in text, os.path.join(dirpath, name)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU: --gpus N > 1 (or a launcher's WORLD_SIZE > 1) exits with a message, before touching a GPU."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for extra_args, extra_env in ((["--gpus", "2"], {}), ([], {"WORLD_SIZE": "2"})):
+        res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), *extra_args], capture_output=True, text=True,
+                             env={**os.environ, **extra_env}, cwd=root, timeout=120)
+        assert res.returncode != 0
+        assert "one GPU" in res.stderr and res.stdout.strip() == ""
