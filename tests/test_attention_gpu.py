@@ -161,15 +161,19 @@ def test_broadcast_masks_and_their_gradient(dtype, mshape, device):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_key_padding_mask_row_broadcast(dtype, device):
-    """[B,1,1,S] additive mask (one row for all queries, row stride 0), as a key-padding mask is given."""
-    B, H, S, D = 2, 3, 256, 64
+@pytest.mark.parametrize("D,S,p", [(64, 256, 0.0), (128, 256, 0.0), (128, 512, 0.0), (128, 512, 0.2)])
+def test_key_padding_mask_row_broadcast(dtype, D, S, p, device):
+    """[B,1,1,S] additive mask (one row for all queries, row stride 0), as a key-padding mask is given. At D = 128 the
+    16-bit dK/dV pass then runs the phased kernel with the mask as one value per key."""
+    B, H = 2, 3
     q, k, v, d_o = _gen((B, H, S, D), 33, dtype)
     mask = torch.zeros(B, 1, 1, S)
-    mask[0, ..., 200:] = float("-inf")
-    mask[1, ..., 131:] = float("-inf")
+    mask[0, ..., S - 56:] = float("-inf")
+    mask[1, ..., S // 2 + 3:] = float("-inf")
     mask += 0.25 * torch.randn(B, 1, 1, S, generator=torch.Generator().manual_seed(34))
-    _check(device, dtype, q, k, v, d_o, mask=mask, tag="key-padding")
+    _check(device, dtype, q, k, v, d_o, mask=mask, dropout_p=p, seed=35 if p else None, tag="key-padding")
+    if dtype == torch.bfloat16:   # the same mask in the operand type
+        _check(device, dtype, q, k, v, d_o, mask=mask.to(dtype), dropout_p=p, seed=35 if p else None, tag="key-padding 16-bit")
 
 
 @pytest.mark.parametrize("dtype,mask_dtype,mshape", [(torch.bfloat16, torch.bfloat16, (2, 3, 256, 256)),

@@ -1283,8 +1283,12 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
 // With DROPOUT only -lse / c is folded into the accumulators: dS = P (Z dP - delta) needs delta beside the dropped dP,
 // so the vector phase reads its 16 row values from the block's slot, and draws the keep decisions of its block (one
 // Philox call per lane, shared inside the quad).
-template <typename T, int D, bool CAUSAL, bool DROPOUT = false>
+// With KEYMASK (kMaskF32 / kMaskT; never with the causal mask): an additive mask that is the same for every query row
+// (row stride 0: a key-padding mask). Lanes own keys here, so the whole mask is one value per lane, read once, and goes
+// into the exponent for free (the multiply by the scale becomes a fused multiply-add).
+template <typename T, int D, bool CAUSAL, bool DROPOUT = false, int KEYMASK = kNoMask>
 __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams p) {
+    static_assert(KEYMASK == kNoMask || !CAUSAL, "a mask excludes the causal variant");
     using Tile = SwzTile<D>;
     constexpr int NW = 8;
     constexpr int kKeys = 128;
@@ -1323,6 +1327,8 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
     const float* lse_base = p.lse + static_cast<int64_t>(bh) * p.S;
     const float* delta_base = p.delta + static_cast<int64_t>(bh) * p.S;
     const float c = p.scale_log2;
+    float key_bias = 0.f;  // mask value of this lane's key, log2 domain
+    if constexpr (KEYMASK != kNoMask) key_bias = mask_at<T, KEYMASK>(p.mask, b * p.ms[0] + hd * p.ms[1] + key) * kLog2e;
 
     f32x16 dk[DH], dv[DH];
 #pragma unroll
@@ -1524,7 +1530,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
 #pragma unroll
                 for (int bb = 0; bb < 4; ++bb) {
                     const int i = 4 * g + bb, j = 4 * g2 + bb;
-                    const float pv = fast_exp2(s[i] * c);
+                    const float pv = KEYMASK != kNoMask ? fast_exp2(fmaf(s[i], c, key_bias)) : fast_exp2(s[i] * c);
                     if constexpr (DROPOUT) {
                         const bool keep = static_cast<int>(dw[bb]) >= p.thr8;
                         pr[j] = keep ? pv * p.zscale : 0.f;
@@ -1745,6 +1751,14 @@ int launch_dkdv_dropout(const KParams& p, hipStream_t stream) {
             if (p.thr8 <= 0) hipLaunchKernelGGL((mfma_dkdv_phased_kernel<T, D, CAUSAL, false>), grid, block, 0, stream, p);
             else hipLaunchKernelGGL((mfma_dkdv_phased_kernel<T, D, CAUSAL, true>), grid, block, 0, stream, p);
             return static_cast<int>(hipGetLastError());
+        }
+        if constexpr (MASK != kNoMask && !CAUSAL) {
+            // a mask that is the same for every query row (a key-padding mask) is one value per key: the phased kernel
+            if (p.ms[2] == 0) {
+                if (p.thr8 <= 0) hipLaunchKernelGGL((mfma_dkdv_phased_kernel<T, D, false, false, MASK>), grid, block, 0, stream, p);
+                else hipLaunchKernelGGL((mfma_dkdv_phased_kernel<T, D, false, true, MASK>), grid, block, 0, stream, p);
+                return static_cast<int>(hipGetLastError());
+            }
         }
         if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dkdv_pair_kernel<T, D, CAUSAL, MASK, true>), grid, block, 0, stream, p);
         else hipLaunchKernelGGL((mfma_dkdv_pair_kernel<T, D, CAUSAL, MASK, false>), grid, block, 0, stream, p);
