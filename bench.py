@@ -206,7 +206,8 @@ def config_figures(dev, with_cpu):
     out = {}
     for name, wl in workloads.WORKLOADS.items():
         pth = Path(wl, dev)
-        ms, pk = run_steps(pth, 3 if name == "C5" else 10, 2)
+        # (enough warm-up steps for the clock to settle after the idle time of the CPU baseline before it)
+        ms, pk = run_steps(pth, 5 if name == "C5" else 30, 2 if name == "C5" else 8)
         peak = PEAK_TFLOPS[_dtype_name(wl.dtype)]
         f = wl.flops() / (pk["fwd"] + pk.get("mask_classes", 0.0)) / 1e9  # (the classification belongs to the forward)
         row = {"workload": describe(wl), "fwd_tflops": round(f, 2), "fwd_frac_of_peak": round(f / peak, 4),
