@@ -56,7 +56,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
     // A mask block of a wave (32 rows x 64 keys) goes through a private LDS region (8 KiB fp32, 4 KiB for a mask of
     // the operand type) when it fits (D = 64): lanes own rows, so direct loads would touch 32 cache lines per
     // instruction, while LDS-direct loads fetch whole rows. Geometry of a 32-row SwzTile<128> / SwzTile<64>.
-    constexpr bool kMaskViaLds = MASK != kNoMask && D == 64;
+    constexpr bool kMaskViaLds = MASK != kNoMask && D == 64;  // (at D = 128 the 4 KiB regions of a 16-bit mask would fit, but the kernel then spills)
     constexpr int kMaskElt = MASK == kMaskF32 ? 4 : 2;
     using MaskTile = std::conditional_t<MASK == kMaskF32, SwzTile<128>, SwzTile<64>>;
     constexpr int kMaskBytes = 32 * MaskTile::kRowBytes;

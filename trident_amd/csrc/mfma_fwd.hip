@@ -52,7 +52,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     // for one of the operand type) when it fits (D = 64): lanes own rows, so direct loads would touch 32 cache
     // lines per instruction, while LDS-direct loads fetch whole rows (256 or 128 bytes) and the swizzled tile is
     // read back 16 or 8 bytes at a time. The region has the geometry of a 32-row SwzTile<128> / SwzTile<64>.
-    constexpr bool kMaskViaLds = MASK != kNoMask && D == 64;
+    constexpr bool kMaskViaLds = MASK != kNoMask && (D == 64 || (MASK == kMaskT && NW == 8));  // (D = 128: 4 KiB regions fit, 8 KiB ones do not)
     constexpr int kMaskElt = MASK == kMaskF32 ? 4 : 2;
     using MaskTile = std::conditional_t<MASK == kMaskF32, SwzTile<128>, SwzTile<64>>;
     constexpr int kMaskBytes = 32 * MaskTile::kRowBytes;

@@ -175,9 +175,9 @@ class Attention(torch.autograd.Function):
             if mask.dtype == torch.bool:
                 if config.reference_limits:
                     raise ValueError("Boolean mask is not supported yet.")
-                # torch's meaning of a boolean attn_mask: True = the key takes part in the attention. The additive mask
-                # is made in fp32: the kernels stage fp32 mask tiles through LDS, 16-bit ones they read element-wise
-                mask = torch.zeros(mask.shape, dtype=torch.float32, device=mask.device).masked_fill_(~mask, float("-inf"))
+                # torch's meaning of a boolean attn_mask: True = the key takes part in the attention (the additive
+                # mask is made in the operand type: half the bytes of an fp32 one for the 16-bit kernels to stream)
+                mask = torch.zeros(mask.shape, dtype=query.dtype, device=mask.device).masked_fill_(~mask, float("-inf"))
 
         seed, offset = _next_seed() if dropout_p > 0.0 else (0, 0)
 
