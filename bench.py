@@ -437,6 +437,8 @@ def main():
                     "(benchmarks/benchmarker.py --scenario attention), one JSON line")
     ap.add_argument("--mode", choices=["forward", "backward"], default="forward")
     ap.add_argument("--dtype", choices=["float32", "float16", "bfloat16"], default="float32")
+    ap.add_argument("--sibling-ops", action="store_true", help="instead of the benchmark: one JSON line with the HBM-bound "
+                    "sibling operations (softmax forward/backward, masked softmax, dropout)")
     ap.add_argument("--ceiling", action="store_true",
                     help="instead of the benchmark: print one JSON line with the MFMA ceiling of this box (random-operand "
                          "MFMA loops, a bf16 GEMM, the C3 kernels)")
@@ -459,6 +461,9 @@ def main():
     w = {**workloads.WORKLOADS, **workloads.EXTRA_WORKLOADS}[a.workload]
     if a.ceiling:
         print(json.dumps({"ceiling": ceiling(dev)}), flush=True)
+        return
+    if a.sibling_ops:
+        print(json.dumps({"sibling_ops": sibling_ops(dev)}), flush=True)
         return
     if a.scenario:
         print(json.dumps({"reference_scenario": reference_scenario(dev, a.mode, a.dtype)}), flush=True)
