@@ -21,7 +21,8 @@
  *     but always fp32). For fp16/bf16 problems the 16-bit matrix-core kernels sum the probabilities as rounded to
  *     that type (the values that multiply V), so lse is accurate to half an ulp of the type times log2(e)
  *     (2.8e-3 for bf16, 3.5e-4 for fp16), not to fp32 precision; the backward calls expect this very lse.
- *     (fp32 problems, and whatever else runs on the fp32 matrix instruction, keep fp32 products and sums throughout.)
+ *     (fp32 problems keep fp32 products and sums throughout; 16-bit problems on the 32-row-tile kernels sum the
+ *     probabilities in fp32 before rounding them for the product with V, so their lse has fp32 accuracy.)
  *   - mask is additive, dtype mask_dtype, logical shape [B, H, S, S] with element strides;
  *     a stride of 0 broadcasts that dimension; the innermost mask stride must be 1.
  *     mask and is_causal are mutually exclusive (trident/operation/attention.py:41-43).
@@ -180,8 +181,9 @@ int64_t tri_attn_mask_classes_size(const TriAttnArgs* args);
 /* Which kernel family a call would run, without launching anything (no counterpart in the reference): pass 0 =
  * tri_attn_fwd, 1 = tri_attn_bwd_dkdv, 2 = tri_attn_bwd_dq on these arguments. Returns 1 for the 16-bit matrix-core
  * (MFMA) kernels (fp16/bf16, D in {64,128}, 16-byte aligned rows; any S without a mask, S a multiple of 128 with
- * one); 2 for the kernels on the fp32 matrix instruction (everything else whose pointers and strides are multiples of
- * four elements: fp32 problems, D in {16,32}, masked lengths that are no multiple of 128; fp32 products and sums);
+ * one); 2 for the 32-row-tile matrix-core kernels (everything else whose pointers and strides are multiples of
+ * four elements: fp32 problems on the fp32 matrix instruction with fp32 products and sums; fp16/bf16 problems with D in
+ * {16,32} or masked lengths that are no multiple of 128 on the 16-bit 32x32x8 instruction);
  * 0 for the general vector-ALU kernels (views that are not aligned so); or a negative TRI_ATTN_E* code. */
 int tri_attn_uses_matrix_cores(const TriAttnArgs* args, int pass);
 

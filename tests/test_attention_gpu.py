@@ -408,9 +408,9 @@ def test_any_length_runs_on_the_matrix_cores(dtype, S, D, variant, device):
     _abi_case(device, dtype, S, D, variant, 600 + S + D, batches=1, heads=3, matrix_cores=True)
 
 
-def test_what_the_16_bit_kernels_leave_runs_on_the_fp32_matrix_instruction(device):
-    """Masked problems of other lengths, fp32 problems and small heads: family 2 (v_mfma_f32_32x32x2_f32) in all
-    three passes."""
+def test_what_the_16_bit_kernels_leave_runs_on_the_32_row_tile_kernels(device):
+    """Masked problems of other lengths, fp32 problems and small heads: family 2 (v_mfma_f32_32x32x2_f32 for fp32 data,
+    the 16-bit 32x32x8 instruction for 16-bit data) in all three passes."""
     _abi_case(device, torch.bfloat16, 200, 64, "mask", 650, matrix_cores=[2, 2, 2])
     _abi_case(device, torch.float32, 256, 64, "plain", 651, matrix_cores=[2, 2, 2])
     _abi_case(device, torch.bfloat16, 256, 32, "causal", 652, matrix_cores=[2, 2, 2])
@@ -419,16 +419,18 @@ def test_what_the_16_bit_kernels_leave_runs_on_the_fp32_matrix_instruction(devic
 @pytest.mark.parametrize("variant", ["plain", "causal", "mask", "mask16", "dropout", "causal+dropout"])
 @pytest.mark.parametrize("dtype,S,D", [(torch.float32, 333, 128), (torch.float32, 200, 64), (torch.float32, 97, 32),
                                        (torch.float32, 70, 16), (torch.float32, 1, 128), (torch.float32, 512, 128),
-                                       (torch.bfloat16, 130, 16), (torch.float16, 260, 32)])
-def test_fp32_matrix_instruction_kernels(dtype, S, D, variant, device):
-    """The kernels on v_mfma_f32_32x32x2_f32 (forward, dQ, dK/dV; the split dK/dV kernel at D = 128) at every head
+                                       (torch.bfloat16, 130, 16), (torch.float16, 260, 32), (torch.float16, 70, 16),
+                                       (torch.bfloat16, 333, 32)])
+def test_32_row_tile_kernels(dtype, S, D, variant, device):
+    """The 32-row-tile kernels (forward, dQ, dK/dV; the split dK/dV kernel at D = 128; fp32 data on
+    v_mfma_f32_32x32x2_f32, 16-bit data on the 32x32x8 instruction of its type) at every head
     size, over lengths with a ragged last tile (and one of a single row), three heads, every mask mode and dropout."""
     if variant == "mask16" and dtype == torch.float32:
         pytest.skip("a 16-bit mask is a mask of the operand type")
     _abi_case(device, dtype, S, D, variant, 700 + S + D, batches=2 if S < 300 else 1, heads=3, matrix_cores=[2, 2, 2])
 
 
-def test_fp32_matrix_instruction_masked_16_bit_lengths(device):
+def test_32_row_tile_kernels_masked_16_bit_lengths(device):
     """16-bit problems the 16-bit kernels leave: a masked length that is no multiple of 128, at D = 64 and 128."""
     _abi_case(device, torch.bfloat16, 200, 128, "mask", 760, heads=3, matrix_cores=[2, 2, 2])
     _abi_case(device, torch.float16, 72, 64, "mask16", 761, heads=3, matrix_cores=[2, 2, 2])

@@ -30,7 +30,7 @@ def _step(lib, tensors, causal, p, backward_entry, delta):
 @pytest.mark.parametrize("dtype,shape,causal,p", [
     (torch.bfloat16, (2, 4, 512, 128), True, 0.0),    # persistent forward, phased dQ with delta, phased dK/dV
     (torch.float16, (1, 3, 256, 64), False, 0.2),     # dropout
-    (torch.float32, (2, 2, 200, 32), True, 0.0),      # kernels on the fp32 matrix instruction, ragged length
+    (torch.float32, (2, 2, 200, 32), True, 0.0),      # 32-row-tile kernels (fp32 matrix instruction), ragged length
 ])
 def test_forward_and_backward_replay_from_a_graph(dtype, shape, causal, p, device):
     lib = _lib.lib()

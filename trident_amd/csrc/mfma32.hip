@@ -1,10 +1,12 @@
-// Attention on the fp32 matrix instruction (v_mfma_f32_32x32x2_f32): fp32 inputs, and every 16-bit problem the
-// 16-bit MFMA kernels do not take (head sizes 16 and 32, masked lengths that are not multiples of 128). Any S >= 1,
-// D in {16, 32, 64, 128}, fp32 / fp16 / bf16 storage, additive mask of any dtype and broadcast, causal mask, dropout.
-// Products and sums are fp32 throughout (the instruction multiplies fp32 exactly), so results agree with the
-// vector-ALU kernels of generic.hip to rounding; those remain for views whose rows are not 4-element aligned.
+// Attention on 32-row tiles, four waves to a workgroup: fp32 inputs (on the fp32 matrix instruction,
+// v_mfma_f32_32x32x2_f32), and every 16-bit problem the 16-bit kernels proper do not take (head sizes 16 and 32, masked
+// lengths that are not multiples of 128; on v_mfma_f32_32x32x8_{f16,bf16_1k}). Any S >= 1, D in {16, 32, 64, 128},
+// fp32 / fp16 / bf16 storage, additive mask of any dtype and broadcast, causal mask, dropout.
+// With fp32 data products and sums are fp32 throughout (the instruction multiplies fp32 exactly), so results agree with
+// the vector-ALU kernels of generic.hip to rounding; those remain for views whose rows are not 4-element aligned. With
+// 16-bit data the inputs enter the matrix pipe as they are and P and dS rounded to their type, sums stay fp32.
 //
-// One 32x32x2 step takes 64 cycles of the matrix pipe for a single 4-byte operand per lane and side, so neither LDS
+// One 32x32x2 step takes 64 cycles of the matrix pipe for a single 4-byte operand per lane and side, so with fp32 data neither LDS
 // bandwidth nor the vector ALU is anywhere near a limit here: the kernels keep it simple. 256 threads = 4 waves; a
 // wave owns 32 rows (queries in forward and dQ, keys in dK/dV) whose operands stay in registers, the other side
 // streams through LDS as fp32 tiles of 32 rows (row stride D + 4 floats: the 16-byte reads of 32 lanes then spread
@@ -16,6 +18,9 @@
 //     that order, and leaves lane (h, l32) with query l32 and keys c_row(r, h);
 //   * O^T += V^T P^T walks the keys in exactly that order, step r using keys {c_row(r, 0), c_row(r, 1)}: the
 //     probabilities are B operands as they stand, no exchange between lanes.
+// Four consecutive steps (one 16-byte piece) are the unit the kernels are written in (quad_t below).
+#include <type_traits>
+
 #include "common.hpp"
 #include "launch.hpp"
 #include "mfma_common.hpp"
@@ -28,6 +33,54 @@ constexpr int kTile32 = 32;         // streamed rows per LDS tile
 
 __device__ __forceinline__ f32x16 mma32(float a, float b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
+// Four consecutive steps of a product's k index as one operand per side. fp32 data keeps the four values and takes
+// four 32x32x2 steps. 16-bit data packs them and takes ONE step of the 16-bit 32x32x8 instruction, whose k index is
+// 4 h + e for value e of half h: the same walk, at eight times the rate; probabilities and dS are then rounded to the
+// 16-bit type on their way into the matrix pipe, exactly as in the 16-bit kernels proper.
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+template <typename T>
+using quad_t = std::conditional_t<sizeof(T) == 4, float4, uint2>;
+template <typename T>
+__device__ __forceinline__ quad_t<T> quad(float4 v) {
+    if constexpr (sizeof(T) == 4) return v;
+    else return uint2{Mma<T>::pack2(v.x, v.y), Mma<T>::pack2(v.z, v.w)};
+}
+template <typename T>
+__device__ __forceinline__ quad_t<T> quad(float a, float b, float c, float d) {
+    return quad<T>(float4{a, b, c, d});
+}
+template <typename T>
+__device__ __forceinline__ f32x16 mma_quad(quad_t<T> a, quad_t<T> b, f32x16 c) {
+    if constexpr (sizeof(T) == 4) {
+        c = mma32(a.x, b.x, c);
+        c = mma32(a.y, b.y, c);
+        c = mma32(a.z, b.z, c);
+        return mma32(a.w, b.w, c);
+    } else if constexpr (std::is_same_v<T, f16_t>) {
+        return __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(f16x4, a), __builtin_bit_cast(f16x4, b), c, 0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(__builtin_bit_cast(s16x4, a), __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
+    }
+}
+// two independent products side by side (fp32: their steps alternate, so that no step waits for the one before it)
+template <typename T>
+__device__ __forceinline__ void mma_quad2(quad_t<T> a0, quad_t<T> b0, f32x16& c0, quad_t<T> a1, quad_t<T> b1, f32x16& c1) {
+    if constexpr (sizeof(T) == 4) {
+        c0 = mma32(a0.x, b0.x, c0);
+        c1 = mma32(a1.x, b1.x, c1);
+        c0 = mma32(a0.y, b0.y, c0);
+        c1 = mma32(a1.y, b1.y, c1);
+        c0 = mma32(a0.z, b0.z, c0);
+        c1 = mma32(a1.z, b1.z, c1);
+        c0 = mma32(a0.w, b0.w, c0);
+        c1 = mma32(a1.w, b1.w, c1);
+    } else {
+        c0 = mma_quad<T>(a0, b0, c0);
+        c1 = mma_quad<T>(a1, b1, c1);
+    }
 }
 
 // four consecutive elements as fp32
@@ -106,17 +159,11 @@ __global__ __launch_bounds__(256, 2) void mfma32_fwd_kernel(const KParams p) {
     const int64_t mrow = p.mask ? b * p.ms[0] + hd * p.ms[1] + qrow_c * p.ms[2] : 0;
 
     // this lane's share of its query row: dims 8 j + 4 h + 0..3
-    float qf[D / 2];
+    quad_t<T> qf[KJ];
     {
         const T* qptr = static_cast<const T*>(p.q) + b * p.qs[0] + hd * p.qs[1] + qrow_c * p.qs[2];
 #pragma unroll
-        for (int j = 0; j < KJ; ++j) {
-            const float4 v = load4(qptr + 8 * j + 4 * h);
-            qf[4 * j + 0] = v.x;
-            qf[4 * j + 1] = v.y;
-            qf[4 * j + 2] = v.z;
-            qf[4 * j + 3] = v.w;
-        }
+        for (int j = 0; j < KJ; ++j) qf[j] = quad<T>(load4(qptr + 8 * j + 4 * h));
     }
     f32x16 oacc[DB];
 #pragma unroll
@@ -142,10 +189,7 @@ __global__ __launch_bounds__(256, 2) void mfma32_fwd_kernel(const KParams p) {
 #pragma unroll
             for (int j = 0; j < KJ; ++j) {
                 const float4 kf = *reinterpret_cast<const float4*>(sK + l32 * LD + 8 * j + 4 * h);
-                s = mma32(kf.x, qf[4 * j + 0], s);
-                s = mma32(kf.y, qf[4 * j + 1], s);
-                s = mma32(kf.z, qf[4 * j + 2], s);
-                s = mma32(kf.w, qf[4 * j + 3], s);
+                s = mma_quad<T>(quad<T>(kf), qf[j], s);
             }
             // scores in the log2 domain: this lane has query qrow and keys k0 + c_row(i, h)
             float x[16];
@@ -188,12 +232,15 @@ __global__ __launch_bounds__(256, 2) void mfma32_fwd_kernel(const KParams p) {
                 }
             }
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float* vrow = sV + c_row(r, h) * LD + l32;
+            for (int g = 0; g < 4; ++g) {  // keys c_row(4 g + e, h) = 8 g + 4 h + e
+                const float* vrow = sV + (8 * g + 4 * h) * LD + l32;
+                const quad_t<T> pq = quad<T>(x[4 * g], x[4 * g + 1], x[4 * g + 2], x[4 * g + 3]);
 #pragma unroll
                 for (int db = 0; db < DB; ++db) {
-                    const float a = (D >= 32 || l32 < D) ? vrow[32 * db] : 0.f;
-                    oacc[db] = mma32(a, x[r], oacc[db]);
+                    const bool in = D >= 32 || l32 < D;
+                    const float* v0 = vrow + 32 * db;
+                    const quad_t<T> a = in ? quad<T>(v0[0], v0[LD], v0[2 * LD], v0[3 * LD]) : quad<T>(0.f, 0.f, 0.f, 0.f);
+                    oacc[db] = mma_quad<T>(a, pq, oacc[db]);
                 }
             }
         }
@@ -246,21 +293,14 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void mfma32_dq_kernel(const 
     const int64_t mrow = p.mask ? b * p.ms[0] + hd * p.ms[1] + qrow_c * p.ms[2] : 0;
     const int64_t dmrow = p.dmask ? b * p.dms[0] + hd * p.dms[1] + qrow_c * p.dms[2] : 0;
 
-    float qf[D / 2], gf[D / 2];
+    quad_t<T> qf[KJ], gf[KJ];
     {
         const T* qptr = static_cast<const T*>(p.q) + b * p.qs[0] + hd * p.qs[1] + qrow_c * p.qs[2];
         const T* gptr = static_cast<const T*>(p.d_o) + b * p.dos[0] + hd * p.dos[1] + qrow_c * p.dos[2];
 #pragma unroll
         for (int j = 0; j < KJ; ++j) {
-            const float4 v = load4(qptr + 8 * j + 4 * h), g = load4(gptr + 8 * j + 4 * h);
-            qf[4 * j + 0] = v.x;
-            qf[4 * j + 1] = v.y;
-            qf[4 * j + 2] = v.z;
-            qf[4 * j + 3] = v.w;
-            gf[4 * j + 0] = g.x;
-            gf[4 * j + 1] = g.y;
-            gf[4 * j + 2] = g.z;
-            gf[4 * j + 3] = g.w;
+            qf[j] = quad<T>(load4(qptr + 8 * j + 4 * h));
+            gf[j] = quad<T>(load4(gptr + 8 * j + 4 * h));
         }
     }
     const float lse = p.lse[static_cast<int64_t>(bh) * p.S + qrow_c];
@@ -289,14 +329,7 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void mfma32_dq_kernel(const 
             for (int j = 0; j < KJ; ++j) {
                 const float4 kf = *reinterpret_cast<const float4*>(sK + l32 * LD + 8 * j + 4 * h);
                 const float4 vf = *reinterpret_cast<const float4*>(sV + l32 * LD + 8 * j + 4 * h);
-                s = mma32(kf.x, qf[4 * j + 0], s);
-                dp = mma32(vf.x, gf[4 * j + 0], dp);
-                s = mma32(kf.y, qf[4 * j + 1], s);
-                dp = mma32(vf.y, gf[4 * j + 1], dp);
-                s = mma32(kf.z, qf[4 * j + 2], s);
-                dp = mma32(vf.z, gf[4 * j + 2], dp);
-                s = mma32(kf.w, qf[4 * j + 3], s);
-                dp = mma32(vf.w, gf[4 * j + 3], dp);
+                mma_quad2<T>(quad<T>(kf), qf[j], s, quad<T>(vf), gf[j], dp);
             }
             // (one branch per tile decides about the mask: a branch per element costs more than the arithmetic it guards)
             float ds[16], mk[16];
@@ -342,12 +375,15 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void mfma32_dq_kernel(const 
                 }
             }
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float* krow = sK + c_row(r, h) * LD + l32;
+            for (int g = 0; g < 4; ++g) {  // keys c_row(4 g + e, h) = 8 g + 4 h + e
+                const float* krow = sK + (8 * g + 4 * h) * LD + l32;
+                const quad_t<T> dq4 = quad<T>(ds[4 * g], ds[4 * g + 1], ds[4 * g + 2], ds[4 * g + 3]);
 #pragma unroll
                 for (int db = 0; db < DB; ++db) {
-                    const float a = (D >= 32 || l32 < D) ? krow[32 * db] : 0.f;
-                    acc[db] = mma32(a, ds[r], acc[db]);
+                    const bool in = D >= 32 || l32 < D;
+                    const float* k0p = krow + 32 * db;
+                    const quad_t<T> a = in ? quad<T>(k0p[0], k0p[LD], k0p[2 * LD], k0p[3 * LD]) : quad<T>(0.f, 0.f, 0.f, 0.f);
+                    acc[db] = mma_quad<T>(a, dq4, acc[db]);
                 }
             }
         }
@@ -401,21 +437,14 @@ __global__ __launch_bounds__(256, D >= 64 ? 1 : 2) void mfma32_dkdv_kernel(const
     const float* delta_base = p.delta + static_cast<int64_t>(bh) * p.S;
     const int64_t mcol = p.mask ? b * p.ms[0] + hd * p.ms[1] + key_c : 0;
 
-    float kf[D / 2], vf[D / 2];
+    quad_t<T> kf[KJ], vf[KJ];
     {
         const T* kptr = static_cast<const T*>(p.k) + b * p.ks[0] + hd * p.ks[1] + key_c * p.ks[2];
         const T* vptr = static_cast<const T*>(p.v) + b * p.vs[0] + hd * p.vs[1] + key_c * p.vs[2];
 #pragma unroll
         for (int j = 0; j < KJ; ++j) {
-            const float4 a = load4(kptr + 8 * j + 4 * h), c = load4(vptr + 8 * j + 4 * h);
-            kf[4 * j + 0] = a.x;
-            kf[4 * j + 1] = a.y;
-            kf[4 * j + 2] = a.z;
-            kf[4 * j + 3] = a.w;
-            vf[4 * j + 0] = c.x;
-            vf[4 * j + 1] = c.y;
-            vf[4 * j + 2] = c.z;
-            vf[4 * j + 3] = c.w;
+            kf[j] = quad<T>(load4(kptr + 8 * j + 4 * h));
+            vf[j] = quad<T>(load4(vptr + 8 * j + 4 * h));
         }
     }
     f32x16 dk[DB], dv[DB];
@@ -454,14 +483,7 @@ __global__ __launch_bounds__(256, D >= 64 ? 1 : 2) void mfma32_dkdv_kernel(const
             for (int j = 0; j < KJ; ++j) {
                 const float4 qa = *reinterpret_cast<const float4*>(sQ + l32 * LD + 8 * j + 4 * h);
                 const float4 ga = *reinterpret_cast<const float4*>(sG + l32 * LD + 8 * j + 4 * h);
-                s = mma32(qa.x, kf[4 * j + 0], s);
-                dp = mma32(ga.x, vf[4 * j + 0], dp);
-                s = mma32(qa.y, kf[4 * j + 1], s);
-                dp = mma32(ga.y, vf[4 * j + 1], dp);
-                s = mma32(qa.z, kf[4 * j + 2], s);
-                dp = mma32(ga.z, vf[4 * j + 2], dp);
-                s = mma32(qa.w, kf[4 * j + 3], s);
-                dp = mma32(ga.w, vf[4 * j + 3], dp);
+                mma_quad2<T>(quad<T>(qa), kf[j], s, quad<T>(ga), vf[j], dp);
             }
             // this lane: its key, rows r0 + c_row(i, h)
             float pr[16], ds[16], mk[16];
@@ -500,14 +522,18 @@ __global__ __launch_bounds__(256, D >= 64 ? 1 : 2) void mfma32_dkdv_kernel(const
                 for (int i = 0; i < 16; ++i) ds[i] = pr[i] * (dp[i] - sDelta[c_row(i, h)]);
             }
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float* grow = sG + c_row(r, h) * LD + l32;
-                const float* qrow = sQ + c_row(r, h) * LD + l32;
+            for (int g = 0; g < 4; ++g) {  // rows c_row(4 g + e, h) = 8 g + 4 h + e
+                const float* grow = sG + (8 * g + 4 * h) * LD + l32;
+                const float* qrow = sQ + (8 * g + 4 * h) * LD + l32;
+                const quad_t<T> p4 = quad<T>(pr[4 * g], pr[4 * g + 1], pr[4 * g + 2], pr[4 * g + 3]);
+                const quad_t<T> s4 = quad<T>(ds[4 * g], ds[4 * g + 1], ds[4 * g + 2], ds[4 * g + 3]);
 #pragma unroll
                 for (int db = 0; db < DB; ++db) {
                     const bool in = D >= 32 || l32 < D;
-                    dv[db] = mma32(in ? grow[32 * db] : 0.f, pr[r], dv[db]);
-                    dk[db] = mma32(in ? qrow[32 * db] : 0.f, ds[r], dk[db]);
+                    const float *g0p = grow + 32 * db, *q0p = qrow + 32 * db;
+                    const quad_t<T> zero = quad<T>(0.f, 0.f, 0.f, 0.f);
+                    mma_quad2<T>(in ? quad<T>(g0p[0], g0p[LD], g0p[2 * LD], g0p[3 * LD]) : zero, p4, dv[db],
+                                 in ? quad<T>(q0p[0], q0p[LD], q0p[2 * LD], q0p[3 * LD]) : zero, s4, dk[db]);
                 }
             }
         }
@@ -630,14 +656,7 @@ __global__ __launch_bounds__(256, 1) void mfma32_dkdv_split_kernel(const KParams
                 const float4 ga = *reinterpret_cast<const float4*>(tG + l32 * LD + 8 * j + 4 * h);
                 const float4 kf = *reinterpret_cast<const float4*>(myK + 8 * j);
                 const float4 vf = *reinterpret_cast<const float4*>(myV + 8 * j);
-                s = mma32(qa.x, kf.x, s);
-                dp = mma32(ga.x, vf.x, dp);
-                s = mma32(qa.y, kf.y, s);
-                dp = mma32(ga.y, vf.y, dp);
-                s = mma32(qa.z, kf.z, s);
-                dp = mma32(ga.z, vf.z, dp);
-                s = mma32(qa.w, kf.w, s);
-                dp = mma32(ga.w, vf.w, dp);
+                mma_quad2<T>(quad<T>(qa), quad<T>(kf), s, quad<T>(ga), quad<T>(vf), dp);
             }
             float pr[16], ds[16], mk[16];
             if (p.mask) {  // (one branch per tile, not one per element)
@@ -674,13 +693,16 @@ __global__ __launch_bounds__(256, 1) void mfma32_dkdv_split_kernel(const KParams
                 for (int i = 0; i < 16; ++i) ds[i] = pr[i] * (dp[i] - sDelta[kTile32 * rh + c_row(i, h)]);
             }
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float* grow = tG + c_row(r, h) * LD + l32;
-                const float* qrow = tQ + c_row(r, h) * LD + l32;
+            for (int g = 0; g < 4; ++g) {  // rows c_row(4 g + e, h) = 8 g + 4 h + e
+                const float* grow = tG + (8 * g + 4 * h) * LD + l32;
+                const float* qrow = tQ + (8 * g + 4 * h) * LD + l32;
+                const quad_t<T> p4 = quad<T>(pr[4 * g], pr[4 * g + 1], pr[4 * g + 2], pr[4 * g + 3]);
+                const quad_t<T> s4 = quad<T>(ds[4 * g], ds[4 * g + 1], ds[4 * g + 2], ds[4 * g + 3]);
 #pragma unroll
                 for (int db = 0; db < DB; ++db) {
-                    dv[db] = mma32(grow[32 * db], pr[r], dv[db]);
-                    dk[db] = mma32(qrow[32 * db], ds[r], dk[db]);
+                    const float *g0p = grow + 32 * db, *q0p = qrow + 32 * db;
+                    mma_quad2<T>(quad<T>(g0p[0], g0p[LD], g0p[2 * LD], g0p[3 * LD]), p4, dv[db],
+                                 quad<T>(q0p[0], q0p[LD], q0p[2 * LD], q0p[3 * LD]), s4, dk[db]);
                 }
             }
         }
