@@ -191,31 +191,51 @@ __global__ __launch_bounds__(256, 2) void mfma32_fwd_kernel(const KParams p) {
                 const float4 kf = *reinterpret_cast<const float4*>(sK + l32 * LD + 8 * j + 4 * h);
                 s = mma_quad<T>(quad<T>(kf), qf[j], s);
             }
-            // scores in the log2 domain: this lane has query qrow and keys k0 + c_row(i, h)
+            // this lane has query qrow and keys k0 + c_row(i, h). One branch per tile picks the work its elements need:
+            // with a mask, scaled scores plus mask values (log2 domain); without one the raw scores, whose scale goes
+            // into the exponent's multiply-add; and only a tile that crosses the diagonal or the end of the sequence
+            // tests its elements for visibility (a branch or a test per element costs more than the arithmetic).
+            const bool edge = k0 + kTile32 > p.S || (p.causal && k0 + kTile32 - 1 > wrow0);
             float x[16];
-            float mx = -INFINITY;
+            float xs = p.scale_log2;  // what x is still to be multiplied by
+            if (p.mask) {
+                xs = 1.f;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int key = k0 + c_row(i, h);
-                float v = s[i] * p.scale_log2;
-                if (p.mask && key < p.S) v = fmaf(load_mask_elem(p.mask, p.mask_dtype, mrow + key), kLog2e, v);
-                const bool visible = key < p.S && (!p.causal || key <= qrow);
-                x[i] = visible ? v : -INFINITY;
-                mx = fmaxf(mx, x[i]);
+                for (int i = 0; i < 16; ++i) {
+                    const int key = k0 + c_row(i, h);
+                    float v = s[i] * p.scale_log2;
+                    if (key < p.S) v = fmaf(load_mask_elem(p.mask, p.mask_dtype, mrow + key), kLog2e, v);
+                    x[i] = key < p.S && (!p.causal || key <= qrow) ? v : -INFINITY;
+                }
+            } else if (edge) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int key = k0 + c_row(i, h);
+                    const bool visible = key < p.S && (!p.causal || key <= qrow);
+                    x[i] = visible ? s[i] : -INFINITY;
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) x[i] = s[i];
             }
-            mx = max_xor32(mx);
+            float mx = x[0];
+#pragma unroll
+            for (int i = 1; i < 16; ++i) mx = fmaxf(mx, x[i]);
+            mx = max_xor32(mx) * xs;
             const float m_new = fmaxf(m, mx);
-            const float m_use = m_new == -INFINITY ? 0.f : m_new;
-            const float alpha = fast_exp2(m - m_use);
-            m = m_new;
-            l *= alpha;  // (each lane sums its own 16 keys of a tile; the two halves meet at the end)
+            if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {  // some row's maximum moved (else every factor is 1)
+                const float alpha = fast_exp2(m - (m_new == -INFINITY ? 0.f : m_new));
+                m = m_new;
+                l *= alpha;  // (each lane sums its own 16 keys of a tile; the two halves meet at the end)
 #pragma unroll
-            for (int db = 0; db < DB; ++db)
+                for (int db = 0; db < DB; ++db)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) oacc[db][i] *= alpha;
+                    for (int i = 0; i < 16; ++i) oacc[db][i] *= alpha;
+            }
+            const float m_use = m == -INFINITY ? 0.f : m;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                x[i] = fast_exp2(x[i] - m_use);
+                x[i] = fast_exp2(fmaf(x[i], xs, -m_use));
                 l += x[i];
             }
             if (p.thr8 > 0) {
@@ -344,11 +364,14 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void mfma32_dq_kernel(const 
                 for (int i = 0; i < 16; ++i) mk[i] = 0.f;
             }
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int key = k0 + c_row(i, h);
-                const float v = fmaf(s[i], p.scale_log2, mk[i]);
-                const bool visible = key < p.S && (!p.causal || key <= qrow);
-                ds[i] = visible ? fast_exp2(v - lse) : 0.f;
+            for (int i = 0; i < 16; ++i) ds[i] = fast_exp2(fmaf(s[i], p.scale_log2, mk[i]) - lse);
+            if (k0 + kTile32 > p.S || (p.causal && k0 + kTile32 - 1 > wrow0)) {  // only such a tile has keys a row does not see
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int key = k0 + c_row(i, h);
+                    const bool visible = key < p.S && (!p.causal || key <= qrow);
+                    ds[i] = visible ? ds[i] : 0.f;
+                }
             }
             if (p.thr8 > 0) {
 #pragma unroll
@@ -419,8 +442,8 @@ __global__ __launch_bounds__(256, D >= 64 ? 1 : 2) void mfma32_dkdv_kernel(const
     constexpr int KJ = D / 8;
     __shared__ __attribute__((aligned(16))) float sQ[kTile32 * LD];
     __shared__ __attribute__((aligned(16))) float sG[kTile32 * LD];
-    __shared__ float sLse[kTile32];
-    __shared__ float sDelta[kTile32];
+    __shared__ __attribute__((aligned(16))) float sLse[kTile32];
+    __shared__ __attribute__((aligned(16))) float sDelta[kTile32];
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
@@ -498,11 +521,15 @@ __global__ __launch_bounds__(256, D >= 64 ? 1 : 2) void mfma32_dkdv_kernel(const
                 for (int i = 0; i < 16; ++i) mk[i] = 0.f;
             }
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int row = r0 + c_row(i, h);
-                const float v = fmaf(s[i], p.scale_log2, mk[i]);
-                const bool visible = row < p.S && key_ok && (!p.causal || key <= row);
-                pr[i] = visible ? fast_exp2(v - sLse[c_row(i, h)]) : 0.f;
+            for (int i = 0; i < 16; ++i) pr[i] = fast_exp2(fmaf(s[i], p.scale_log2, mk[i]) - sLse[c_row(i, h)]);
+            // only a tile at the end of the sequence (rows or keys) or on the diagonal has elements that do not exist
+            if (r0 + kTile32 > p.S || wkey0 + 32 > p.S || (p.causal && r0 < wkey0 + 31)) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int row = r0 + c_row(i, h);
+                    const bool visible = row < p.S && key_ok && (!p.causal || key <= row);
+                    pr[i] = visible ? pr[i] : 0.f;
+                }
             }
             if (p.thr8 > 0) {
 #pragma unroll
@@ -574,8 +601,8 @@ __global__ __launch_bounds__(256, 1) void mfma32_dkdv_split_kernel(const KParams
     __shared__ __attribute__((aligned(16))) float sV[kKeys * LD];
     __shared__ __attribute__((aligned(16))) float sQ[2 * kTile32 * LD];  // tiles 2 u and 2 u + 1
     __shared__ __attribute__((aligned(16))) float sG[2 * kTile32 * LD];
-    __shared__ float sLse[2 * kTile32];
-    __shared__ float sDelta[2 * kTile32];
+    __shared__ __attribute__((aligned(16))) float sLse[2 * kTile32];
+    __shared__ __attribute__((aligned(16))) float sDelta[2 * kTile32];
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int kb = wave & 1, rh = wave >> 1;
@@ -670,11 +697,14 @@ __global__ __launch_bounds__(256, 1) void mfma32_dkdv_split_kernel(const KParams
                 for (int i = 0; i < 16; ++i) mk[i] = 0.f;
             }
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int row = r0 + c_row(i, h);
-                const float v = fmaf(s[i], p.scale_log2, mk[i]);
-                const bool visible = row < p.S && key_ok && (!p.causal || key <= row);
-                pr[i] = visible ? fast_exp2(v - sLse[kTile32 * rh + c_row(i, h)]) : 0.f;
+            for (int i = 0; i < 16; ++i) pr[i] = fast_exp2(fmaf(s[i], p.scale_log2, mk[i]) - sLse[kTile32 * rh + c_row(i, h)]);
+            if (r0 + kTile32 > p.S || wkey0 + 32 > p.S || (p.causal && r0 < wkey0 + 31)) {  // (as in the kernel above)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int row = r0 + c_row(i, h);
+                    const bool visible = row < p.S && key_ok && (!p.causal || key <= row);
+                    pr[i] = visible ? pr[i] : 0.f;
+                }
             }
             if (p.thr8 > 0) {
 #pragma unroll

@@ -44,9 +44,11 @@ WORKLOADS = {
     "C5": Workload("C5", torch.bfloat16, 1, 32, 16384, 128, is_causal=True, dropout_p=0.1, sigma_qkv=0.5, seed=1005),
 }
 
-# Beyond the five benchmark configurations: C3's shape in fp32 (the kernels on the fp32 matrix instruction at a real size).
+# Beyond the five benchmark configurations: C3's shape in fp32 (the kernels on the fp32 matrix instruction at a real
+# size) and a 16-bit problem with a small head (the same kernels on the 16-bit 32x32x8 instruction).
 EXTRA_WORKLOADS = {
     "F3": Workload("F3", torch.float32, 2, 16, 4096, 128, is_causal=True, seed=1103),
+    "H32": Workload("H32", torch.bfloat16, 8, 16, 2048, 32, is_causal=True, seed=1132),
 }
 
 
