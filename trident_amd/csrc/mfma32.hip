@@ -352,19 +352,20 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void mfma32_dq_kernel(const 
                 mma_quad2<T>(quad<T>(kf), qf[j], s, quad<T>(vf), gf[j], dp);
             }
             // (one branch per tile decides about the mask: a branch per element costs more than the arithmetic it guards)
-            float ds[16], mk[16];
+            float ds[16];
             if (p.mask) {
+                float mk[16];
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int key = k0 + c_row(i, h);
                     mk[i] = key < p.S ? load_mask_elem(p.mask, p.mask_dtype, mrow + key) * kLog2e : 0.f;
                 }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) ds[i] = fast_exp2(fmaf(s[i], p.scale_log2, mk[i]) - lse);
             } else {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) mk[i] = 0.f;
+                for (int i = 0; i < 16; ++i) ds[i] = fast_exp2(fmaf(s[i], p.scale_log2, -lse));
             }
-#pragma unroll
-            for (int i = 0; i < 16; ++i) ds[i] = fast_exp2(fmaf(s[i], p.scale_log2, mk[i]) - lse);
             if (k0 + kTile32 > p.S || (p.causal && k0 + kTile32 - 1 > wrow0)) {  // only such a tile has keys a row does not see
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
@@ -509,19 +510,20 @@ __global__ __launch_bounds__(256, D >= 64 ? 1 : 2) void mfma32_dkdv_kernel(const
                 mma_quad2<T>(quad<T>(qa), kf[j], s, quad<T>(ga), vf[j], dp);
             }
             // this lane: its key, rows r0 + c_row(i, h)
-            float pr[16], ds[16], mk[16];
+            float pr[16], ds[16];
             if (p.mask) {  // (one branch per tile, not one per element)
+                float mk[16];
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int row = r0 + c_row(i, h);
                     mk[i] = row < p.S ? load_mask_elem(p.mask, p.mask_dtype, mcol + row * p.ms[2]) * kLog2e : 0.f;
                 }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) pr[i] = fast_exp2(fmaf(s[i], p.scale_log2, mk[i]) - sLse[c_row(i, h)]);
             } else {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) mk[i] = 0.f;
+                for (int i = 0; i < 16; ++i) pr[i] = fast_exp2(fmaf(s[i], p.scale_log2, -sLse[c_row(i, h)]));
             }
-#pragma unroll
-            for (int i = 0; i < 16; ++i) pr[i] = fast_exp2(fmaf(s[i], p.scale_log2, mk[i]) - sLse[c_row(i, h)]);
             // only a tile at the end of the sequence (rows or keys) or on the diagonal has elements that do not exist
             if (r0 + kTile32 > p.S || wkey0 + 32 > p.S || (p.causal && r0 < wkey0 + 31)) {
 #pragma unroll
@@ -685,19 +687,20 @@ __global__ __launch_bounds__(256, 1) void mfma32_dkdv_split_kernel(const KParams
                 const float4 vf = *reinterpret_cast<const float4*>(myV + 8 * j);
                 mma_quad2<T>(quad<T>(qa), quad<T>(kf), s, quad<T>(ga), quad<T>(vf), dp);
             }
-            float pr[16], ds[16], mk[16];
+            float pr[16], ds[16];
             if (p.mask) {  // (one branch per tile, not one per element)
+                float mk[16];
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int row = r0 + c_row(i, h);
                     mk[i] = row < p.S ? load_mask_elem(p.mask, p.mask_dtype, mcol + row * p.ms[2]) * kLog2e : 0.f;
                 }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) pr[i] = fast_exp2(fmaf(s[i], p.scale_log2, mk[i]) - sLse[kTile32 * rh + c_row(i, h)]);
             } else {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) mk[i] = 0.f;
+                for (int i = 0; i < 16; ++i) pr[i] = fast_exp2(fmaf(s[i], p.scale_log2, -sLse[kTile32 * rh + c_row(i, h)]));
             }
-#pragma unroll
-            for (int i = 0; i < 16; ++i) pr[i] = fast_exp2(fmaf(s[i], p.scale_log2, mk[i]) - sLse[kTile32 * rh + c_row(i, h)]);
             if (r0 + kTile32 > p.S || wkey0 + 32 > p.S || (p.causal && r0 < wkey0 + 31)) {  // (as in the kernel above)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
