@@ -4,6 +4,7 @@ The first three tests are the reference's own (tests/test_attention.py:22-116) w
 inputs, the oracle in place of the run-time PyTorch call, and the tighter tolerance of this
 build (fp32 atol 1e-4 instead of 1e-2)."""
 import math
+import os
 
 import numpy as np
 import pytest
@@ -481,10 +482,13 @@ def _random_cases(count, seed):
     return cases
 
 
-@pytest.mark.parametrize("dtype,S,D,variant,batches,heads,seed", _random_cases(48, 20240611))
+@pytest.mark.parametrize("dtype,S,D,variant,batches,heads,seed",
+                         _random_cases(int(os.environ.get("TRI_RANDOM_CASES", "48")),
+                                       int(os.environ.get("TRI_RANDOM_SEED", "20240611"))))
 def test_random_problems(dtype, S, D, variant, batches, heads, seed, device):
     """A fixed pseudo-random sample of (dtype, length, head size, mask mode, dropout, batch, heads): whatever kernel
-    family the dispatch picks, forward, LSE, delta and the three gradients match the oracle."""
+    family the dispatch picks, forward, LSE, delta and the three gradients match the oracle. TRI_RANDOM_CASES and
+    TRI_RANDOM_SEED in the environment draw a larger or another sample."""
     _abi_case(device, dtype, S, D, variant, seed, batches=batches, heads=heads)
 
 
