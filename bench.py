@@ -381,11 +381,12 @@ def ceiling(dev):
     for matrix, mname in ((0, "bf16_32x32x16"), (1, "fp32_32x32x2")):
         for valu, vname in ((0, "fma"), (1, "exp2"), (2, "fma_max_exp2")):
             row = {}
-            for who, wname in ((1, "matrix_ms"), (2, "vector_ms"), (3, "both_ms")):
+            for who, wname in ((1, "matrix_ms"), (2, "vector_ms"), (3, "both_ms"), (4, "same_wave_ms")):
                 row[wname] = round(timed(lambda: _lib.check(lib.tri_attn_probe_coexec(
                     matrix, valu, who, cus, 2000, operands.data_ptr(), out.data_ptr(),
                     torch.cuda.current_stream().cuda_stream)), 3), 3)
             row["hidden_fraction_of_vector_work"] = round((row["matrix_ms"] + row["vector_ms"] - row["both_ms"]) / row["vector_ms"], 3)
+            row["hidden_fraction_same_wave"] = round((row["matrix_ms"] + row["vector_ms"] - row["same_wave_ms"]) / row["vector_ms"], 3)
             co[mname + "+" + vname] = row
     res["coexecution"] = co
     n = 8192

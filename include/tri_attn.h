@@ -206,7 +206,8 @@ int tri_attn_probe_mfma(int mode, int workgroups, int iters, const void* operand
 /* Calibration, no counterpart in the reference: does vector-ALU work of one wave run in the shadow of another wave's
  * MFMAs on the same SIMD? Waves 0-3 of each 512-thread workgroup issue 16 MFMAs per loop trip (matrix 0:
  * v_mfma_f32_32x32x16_bf16, 1: v_mfma_f32_32x32x2_f32), waves 4-7 work on 32 values per lane per trip (valu 0: one fma
- * each, 1: one exp2 each, 2: fma + max + exp2 each). who: 1 = the matrix waves only, 2 = the vector waves only, 3 = both.
+ * each, 1: one exp2 each, 2: fma + max + exp2 each). who: 1 = the matrix waves only, 2 = the vector waves only, 3 = both;
+ * 4 = waves 0-3 do both kinds of work themselves (two values' vector work after each matrix step), waves 4-7 nothing.
  * operands: 10 * 512 * 16 bytes; out: workgroups * 512 floats. Used by bench.py --ceiling. */
 int tri_attn_probe_coexec(int matrix, int valu, int who, int workgroups, int iters, const void* operands, float* out,
                           void* stream);

@@ -80,12 +80,13 @@ __global__ __launch_bounds__(kProbeThreads) void probe_kernel(const u32x4* __res
 // Do vector-ALU instructions of one wave run in the shadow of another wave's MFMAs on the same SIMD? Waves 0-3 of a
 // workgroup (one per SIMD) run MFMAs (MATRIX 0: v_mfma_f32_32x32x16_bf16, 1: v_mfma_f32_32x32x2_f32; 16 per loop trip
 // on 4 accumulators), waves 4-7 run vector work on 32 independent values per lane (VALU 0: one fma each; 1: one exp2 each;
-// 2: fma, max, exp2 each - a softmax's mix). `who` selects which group works: 1 matrix only, 2 vector only, 3 both.
+// 2: fma, max, exp2 each - a softmax's mix). `who` selects which group works: 1 matrix only, 2 vector only, 3 both; 4 = waves 0-3 do both kinds of work themselves (two values'
+// vector work after each matrix step) and waves 4-7 nothing.
 template <int MATRIX, int VALU>
 __global__ __launch_bounds__(kProbeThreads) void coexec_kernel(const u32x4* __restrict__ operands, float* out, int iters, int who) {
     const int tid = threadIdx.x, group = tid >> 8;
     float acc = 0.f;
-    if ((who & 1) && group == 0) {
+    if (who != 4 && (who & 1) && group == 0) {
         f32x16 c[4] = {zero16(), zero16(), zero16(), zero16()};
         const u32x4 a = operands[tid], b = operands[kProbeThreads + tid];
         for (int it = 0; it < iters; ++it) {
@@ -98,7 +99,37 @@ __global__ __launch_bounds__(kProbeThreads) void coexec_kernel(const u32x4* __re
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc += (c[0][i] + c[1][i]) + (c[2][i] + c[3][i]);
     }
-    if ((who & 2) && group == 1) {
+    if (who == 4 && group == 0) {  // both kinds of work in the SAME wave: each matrix step followed by two values' vector work
+        f32x16 c[4] = {zero16(), zero16(), zero16(), zero16()};
+        const u32x4 a = operands[tid], b = operands[kProbeThreads + tid];
+        float x[32];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const u32x4 v = operands[2 * kProbeThreads + i * kProbeThreads + tid];
+            x[4 * i + 0] = __builtin_bit_cast(float, v.x) * 1e-3f;
+            x[4 * i + 1] = __builtin_bit_cast(float, v.y) * 1e-3f;
+            x[4 * i + 2] = __builtin_bit_cast(float, v.z) * 1e-3f;
+            x[4 * i + 3] = __builtin_bit_cast(float, v.w) * 1e-3f;
+        }
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                if constexpr (MATRIX == 0) c[j & 3] = Mma<bf16_t>::run(a, b, c[j & 3]);
+                else c[j & 3] = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, a.x), __builtin_bit_cast(float, b.x), c[j & 3], 0, 0, 0);
+#pragma unroll
+                for (int i = 2 * j; i < 2 * j + 2; ++i) {
+                    if constexpr (VALU == 0) x[i] = fmaf(x[i], 0.999f, 0.001f);
+                    else if constexpr (VALU == 1) x[i] = fast_exp2(x[i] * 0.5f);
+                    else x[i] = fast_exp2(fmaxf(fmaf(x[i], 0.999f, 0.001f), 0.25f) - 1.f);
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc += (c[0][i] + c[1][i]) + (c[2][i] + c[3][i]);
+#pragma unroll
+        for (int i = 0; i < 32; ++i) acc += x[i];
+    }
+    if (who != 4 && (who & 2) && group == 1) {
         float x[32];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -130,7 +161,7 @@ using namespace tri;
 extern "C" int tri_attn_probe_coexec(int matrix, int valu, int who, int workgroups, int iters, const void* operands,
                                      float* out, void* stream) {
     if (operands == nullptr || out == nullptr) return TRI_ATTN_ENULL;
-    if (workgroups <= 0 || iters <= 0 || matrix < 0 || matrix > 1 || valu < 0 || valu > 2 || who < 1 || who > 3) return TRI_ATTN_ESHAPE;
+    if (workgroups <= 0 || iters <= 0 || matrix < 0 || matrix > 1 || valu < 0 || valu > 2 || who < 1 || who > 4) return TRI_ATTN_ESHAPE;
     const dim3 grid(workgroups), block(kProbeThreads);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const u32x4* ops = static_cast<const u32x4*>(operands);
