@@ -142,13 +142,19 @@ def test_shapes(dtype, S, D, variant, device):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_strided_inputs(dtype, device):
-    """[B,S,H,D] storage viewed as [B,H,S,D]: rows of one head are H*D apart."""
-    B, H, S, D = 2, 4, 256, 64
+@pytest.mark.parametrize("S,D,causal", [(256, 64, True), (512, 128, False), (200, 128, True), (333, 32, False)])
+def test_strided_inputs(dtype, S, D, causal, device):
+    """[B,S,H,D] storage viewed as [B,H,S,D]: rows of one head are H*D apart. Through the phased 16-bit kernels, their
+    variants for other lengths, and the 32-row-tile kernels (fp32; head size 32)."""
+    B, H = 2, 4
     g = torch.Generator().manual_seed(21)
     q, k, v, d_o = [torch.randn(B, S, H, D, generator=g).to(dtype).transpose(1, 2) for _ in range(4)]
     assert not q.is_contiguous()
-    _check(device, dtype, q, k, v, d_o, is_causal=True, tag="strided")
+    trident.config.reference_limits = S in (256, 512)
+    try:
+        _check(device, dtype, q, k, v, d_o, is_causal=causal, tag=f"strided S={S} D={D}")
+    finally:
+        trident.config.reference_limits = True
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
