@@ -8,6 +8,12 @@ backward pre-pass (delta), dK/dV and dQ, called through the C ABI on tensors tha
 resident in HBM. The default workload is C3 (bf16, causal, B=2 H=16 S=4096 D=128), the one the
 headline metric is quoted on. Rank 0 prints ONE JSON line on stdout; --report additionally
 prints forward and forward+backward figures for all five configurations on stderr.
+
+Order of a run: the CPU baselines first (the GPU idles meanwhile), then the per-configuration and
+sibling-operation figures, and the headline region (W warm-up steps, K timed steps) LAST, directly
+after them. An MI355X that has idled takes some tens of milliseconds of load to raise its clocks: timed
+right after start-up, 5 warm-up steps (3 ms) are not enough and the same K steps take about 12 % longer
+(that figure is reported as `cold_start`). `value` is the sustained rate.
 """
 import argparse
 import ctypes
@@ -23,15 +29,27 @@ if ROOT not in sys.path:
 PEAK_TFLOPS = {"bf16": 2516.6, "fp16": 2516.6, "fp32": 157.3}  # MI355X dense MFMA peaks (256 CU x 2.4 GHz)
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (see profiles/); None where not measured.
-MEASURED_TRAFFIC = {
-    # (workload, kernel): bytes read + written per launch (profiles/c3_hbm_traffic.txt)
-    ("C3", "fwd"): int((143.5 + 32.5) * 2**20),
-    ("C3", "bwd_dkdv"): int((211.6 + 64.0) * 2**20),
-    ("C3", "bwd_dq"): int((246.0 + 32.5) * 2**20),  # with the delta pre-pass folded in (reads O too)
-    ("C3", "bwd_delta"): int((64.0 + 0.5) * 2**20),
-}
+
+
+def measured_traffic(workload, kernel):
+    """HBM bytes (read + written) per launch of a kernel as measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE:
+    parsed from the summary profiles/<workload>_hbm_traffic.txt (columns: kernel, FETCH_SIZE KiB, scaled read MiB,
+    WRITE_SIZE KiB, written MiB); None where no summary covers the kernel."""
+    path = os.path.join(ROOT, "profiles", f"{workload.lower()}_hbm_traffic.txt")
+    if not os.path.exists(path):
+        return None
+    for line in open(path):
+        if not line.startswith("# " + kernel + " "):
+            continue
+        nums = []
+        for tok in line.split():
+            try:
+                nums.append(float(tok))
+            except ValueError:
+                pass
+        if len(nums) >= 4:
+            return int((nums[1] + nums[3]) * 2**20)
+    return None
 
 
 def _dtype_name(dtype):
@@ -108,7 +126,11 @@ class Path:
 
 
 def run_steps(path, steps, warmup):
-    """Returns (ms per step by wall clock, {kernel: avg ms} from HIP events on the launch stream)."""
+    """Returns (ms per step by wall clock, {kernel: avg ms} from HIP events on the launch stream).
+
+    Every timed step brackets ONE of its kernels with a pair of events, step s the kernel s mod n: an event record is
+    a packet of its own in the queue, and a pair around every kernel of every step makes the step 2-3 % longer than
+    the same launches back to back. A kernel's average is over the steps that bracketed it."""
     import torch
 
     for _ in range(warmup):
@@ -116,19 +138,30 @@ def run_steps(path, steps, warmup):
             fn()
     torch.cuda.synchronize()
     n = len(path.kernels)
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(n + 1)] for _ in range(steps)]
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for s in range(steps):
-        events[s][0].record()
         for i, (_, fn) in enumerate(path.kernels):
-            fn()
-            events[s][i + 1].record()
+            if i == s % n:
+                events[s][0].record()
+                fn()
+                events[s][1].record()
+            else:
+                fn()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     per_kernel = {}
-    for i, (name, _) in enumerate(path.kernels):
-        per_kernel[name] = sum(events[s][i].elapsed_time(events[s][i + 1]) for s in range(steps)) / steps
+    for i, (name, fn) in enumerate(path.kernels):
+        samples = [events[s][0].elapsed_time(events[s][1]) for s in range(steps) if s % n == i]
+        if not samples:  # fewer steps than kernels: one more launch of this kernel, outside the timed region
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            torch.cuda.synchronize()
+            samples = [e0.elapsed_time(e1)]
+        per_kernel[name] = sum(samples) / len(samples)
     return wall_ms, per_kernel
 
 
@@ -477,10 +510,27 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     path = Path(w, dev)
+    flops_step = w.flops(w.backward)
+    # right after start-up, on a clock that is still rising from idle: reported, not the headline
+    cold_ms, _ = run_steps(path, a.steps, a.warmup)
+    extras = {"cold_start": {"ms_per_step": round(cold_ms, 5), "tflops": round(flops_step / cold_ms / 1e9, 1),
+                             "note": "the same W + K steps as the first GPU work of the process, before the clock has settled"}}
+    if not a.no_cpu:
+        extras["cpu_baseline"] = cpu_baseline(w)
+    if not a.no_configs:
+        for key, leg in (("configs", lambda: config_figures(dev, not a.no_cpu)), ("sibling_ops", lambda: sibling_ops(dev))):
+            try:
+                extras[key] = leg()
+            except Exception as e:  # (the headline below must not depend on the other legs)
+                extras[key] = {"error": f"{type(e).__name__}: {e}"}
+    op_steps, op_warmup = max(a.steps, 100), max(a.warmup, 20)
+    op_ms = operator_ms(w, dev, op_steps, op_warmup)
+    extras["operator_api"] = {"ms_per_step": round(op_ms, 5), "tflops": round(flops_step / op_ms / 1e9, 1), "steps": op_steps,
+                              "warmup": op_warmup, "note": "same step through function.scaled_dot_product_attention + autograd"}
+    # the headline region, directly after sustained load on the same workload
     wall_ms, per_kernel = run_steps(path, a.steps, a.warmup)
     dname = _dtype_name(w.dtype)
     peak = PEAK_TFLOPS[dname]
-    flops_step = w.flops(w.backward)
     value = flops_step / wall_ms / 1e9
     fwd_tf = w.flops() / (per_kernel["fwd"] + per_kernel.get("mask_classes", 0.0)) / 1e9
 
@@ -494,7 +544,7 @@ def main():
         "peak": peak,
         "unit": "TFLOP/s",
         "frac": round(achieved / peak, 4),
-        "traffic": MEASURED_TRAFFIC.get((w.name, dominant)),
+        "traffic": measured_traffic(w.name, dominant),
         "avg_launch_ms": round(per_kernel[dominant], 5),
     }
     result = {
@@ -524,14 +574,7 @@ def main():
         gbs = nbytes / per_kernel["bwd_delta"] / 1e6
         result["delta_prepass"] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                    "frac": round(gbs / HBM_PEAK_GBS, 4)}
-    op_ms = operator_ms(w, dev, a.steps, a.warmup)
-    result["operator_api"] = {"ms_per_step": round(op_ms, 5), "tflops": round(flops_step / op_ms / 1e9, 1),
-                              "note": "same step through function.scaled_dot_product_attention + autograd"}
-    if not a.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(w)
-    if not a.no_configs:
-        result["configs"] = config_figures(dev, not a.no_cpu)
-        result["sibling_ops"] = sibling_ops(dev)
+    result.update(extras)
     print(json.dumps(result), flush=True)
 
     if a.report:

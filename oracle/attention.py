@@ -178,8 +178,8 @@ def attention_rows(q_rows, k, v, d_out_rows, row0, bh, mask_rows=None, dropout_p
 
 def operand_abs_sums(q, k, v, d_out, mask=None, dropout_p=0.0, is_causal=False, scale=None, seed=0, offset=0, o=None):
     """Sum of |terms| of the contractions whose left operand a 16-bit matrix-core kernel must round
-    (P for O and dV, dS for dQ and dK): A_O = |PZ| |V|, A_dV = |PZ|^T |dO|, A_dQ = scale |dS| |K|,
-    A_dK = scale |dS|^T |Q|.  Rounding P or dS to a type with unit roundoff u perturbs each output by
+    (P for O and dV, dS for dQ and dK): A_O = |PZ| |V|, A_dV = |PZ|^T |dO|, A_dQ = |scale| |dS| |K|,
+    A_dK = |scale| |dS|^T |Q|.  Rounding P or dS to a type with unit roundoff u perturbs each output by
     at most u * A, whatever the kernel; the parity tests add that bound to the stated atol."""
     q, k, v, d_out = [np.asarray(x, dtype=np.float64) for x in (q, k, v, d_out)]
     B, H, S, D = q.shape
@@ -200,8 +200,8 @@ def operand_abs_sums(q, k, v, d_out, mask=None, dropout_p=0.0, is_causal=False, 
             ds = np.abs(p * (dp - dlt[:, None]))
             a_o[b, h] = pz @ np.abs(v[b, h])
             a_dv[b, h] = pz.T @ np.abs(d_out[b, h])
-            a_dq[b, h] = scale * (ds @ np.abs(k[b, h]))
-            a_dk[b, h] = scale * (ds.T @ np.abs(q[b, h]))
+            a_dq[b, h] = abs(scale) * (ds @ np.abs(k[b, h]))
+            a_dk[b, h] = abs(scale) * (ds.T @ np.abs(q[b, h]))
     return a_o, a_dq, a_dk, a_dv
 
 

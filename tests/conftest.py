@@ -19,3 +19,19 @@ def device():
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     return torch.device("cuda:0")
+
+
+def pytest_sessionfinish(session, exitstatus):
+    """After a session that compared GPU results with the oracle: the margins of every comparison, as text."""
+    from tests import parity
+
+    if not any(r["elements"] for r in parity.MARGINS):
+        return
+    import torch
+
+    if not torch.cuda.is_available():
+        return
+    out = os.path.join(ROOT, "gpurun_out")
+    os.makedirs(out, exist_ok=True)
+    with open(os.path.join(out, "parity_margins.txt"), "w") as f:
+        f.write(parity.margins_summary())

@@ -1,4 +1,6 @@
 """Shared helpers of the parity tests: oracle calls on torch tensors and the comparison rule."""
+import os
+
 import numpy as np
 import torch
 
@@ -21,6 +23,19 @@ def to64(t):
     return None if t is None else t.detach().cpu().to(torch.float64).numpy()
 
 
+# Every comparison leaves a record here: how far beyond the plain atol the two documented additions (storage rounding
+# of a 16-bit result, rounding of the 16-bit MFMA operand) had to stretch. tests/conftest.py writes the summary of a
+# GPU session to gpurun_out/parity_margins.txt, and `close` itself bounds both: of a 16-bit comparison at most
+# OVER_ATOL_FRACTION of the elements may lie above the plain atol, and none further than OVER_ATOL_FACTOR times
+# it (fp32 comparisons: none at all above 1e-4 + 1e-5 |x|, which the rule already says). The bounds sit just above
+# what a recorded session shows (profiles/parity_margins.txt: of 331 million bf16 elements five lie above the plain
+# atol, the worst at 1.18 times it; worst fraction of one comparison 2.3e-5, in dV under dropout), so a defect of a few
+# 1e-2 on an ill-conditioned sum no longer hides behind the operand allowance.
+MARGINS = []
+OVER_ATOL_FRACTION = 1e-4
+OVER_ATOL_FACTOR = 2.0
+
+
 def close(actual: torch.Tensor, expected: np.ndarray, dtype, what="", abs_sum=None, stats=None):
     a = actual.detach().cpu().to(torch.float64).numpy()
     e = np.asarray(expected, dtype=np.float64)
@@ -34,19 +49,53 @@ def close(actual: torch.Tensor, expected: np.ndarray, dtype, what="", abs_sum=No
     tol = np.where(np.isfinite(tol), tol, np.inf)
     bad = ~(err <= tol)
     bad &= ~((a == e) & ~np.isnan(a))  # equal infinities
+    # how much of the tolerance beyond the plain atol was needed (quantifies the two documented additions); the
+    # storage rounding of the expected value itself (half an ulp of a 16-bit result) is not counted as excess
+    finite = np.isfinite(err)
+    excess = np.where(finite, err - RTOL[dtype] * np.abs(np.where(np.isfinite(e), e, 0.0)), 0.0)
+    over = finite & (excess > ATOL[dtype])
+    record = dict(what=what, dtype=str(dtype).replace("torch.", ""), elements=int(a.size), over_atol=int(over.sum()),
+                  max_err=float(np.nanmax(err[finite])) if finite.any() else 0.0,
+                  max_over_atol=float((excess[over] / ATOL[dtype]).max()) if over.any() else 0.0)
+    MARGINS.append(record)
     if stats is not None:
-        # how much of the tolerance beyond the plain atol was needed (quantifies the two documented additions)
-        finite = np.isfinite(err)
-        over = finite & (err > ATOL[dtype])
-        stats.update(elements=int(a.size), over_atol=int(over.sum()), max_err=float(np.nanmax(err)) if err.size else 0.0,
-                     max_over_atol=float((err[over] / ATOL[dtype]).max()) if over.any() else 0.0)
+        stats.update(record)
     if bad.any():
         idx = np.unravel_index(np.argmax(np.where(bad, err, 0)), a.shape)
         raise AssertionError(
             f"{what}: {bad.sum()} of {a.size} elements off; worst at {idx}: got {a[idx]!r}, want {e[idx]!r}, "
             f"max abs err {np.nanmax(err):.3e}"
         )
+    if os.environ.get("TRI_PARITY_RECORD_ONLY"):  # (a session that only gathers the margins)
+        return float(np.nanmax(err)) if err.size else 0.0
+    if a.size >= 4096:  # (a fraction means little on a handful of elements)
+        assert record["over_atol"] <= OVER_ATOL_FRACTION * a.size, \
+            f"{what}: {record['over_atol']} of {a.size} elements needed more than the plain atol {ATOL[dtype]}"
+    assert record["max_over_atol"] <= OVER_ATOL_FACTOR, \
+        f"{what}: an element is {record['max_over_atol']:.2f} x the plain atol {ATOL[dtype]} off (after its storage rounding)"
     return float(np.nanmax(err)) if err.size else 0.0
+
+
+def margins_summary():
+    """Text summary of MARGINS: per dtype the totals and the worst comparisons."""
+    lines = ["# comparisons against the fp64 oracle in this session: elements whose error exceeded the plain atol",
+             "# (fp32 1e-4, fp16 / bf16 1e-2) after the storage rounding of a 16-bit result was taken off",
+             f"# bounds enforced by tests/parity.py: fraction <= {OVER_ATOL_FRACTION:g} per comparison of >= 4096 elements, "
+             f"worst element <= {OVER_ATOL_FACTOR:g} x atol"]
+    for dt in ("float32", "float16", "bfloat16"):
+        rows = [r for r in MARGINS if r["dtype"] == dt]
+        if not rows:
+            continue
+        n = sum(r["elements"] for r in rows)
+        over = sum(r["over_atol"] for r in rows)
+        lines.append(f"{dt}: {len(rows)} comparisons, {n} elements, {over} above the plain atol ({over / max(n, 1):.2e}); "
+                     f"worst element {max(r['max_over_atol'] for r in rows):.2f} x atol; largest error {max(r['max_err'] for r in rows):.3e}")
+        worst = sorted(rows, key=lambda r: (-r["over_atol"] / max(r["elements"], 1), -r["max_over_atol"]))[:8]
+        for r in worst:
+            if r["over_atol"]:
+                lines.append(f"    {r['what'] or '(unnamed)'}: {r['over_atol']} of {r['elements']} ({r['over_atol'] / r['elements']:.2e}), "
+                             f"worst {r['max_over_atol']:.2f} x atol, max err {r['max_err']:.3e}")
+    return "\n".join(lines) + "\n"
 
 
 # The matrix-core forward kernels take the softmax denominator over the probabilities ROUNDED to the 16-bit

@@ -67,6 +67,17 @@ def test_status_codes_without_gpu():
     big.B, big.H, big.S, big.D = 1, 64, _lib.NOALLOC_MAX_ROWS // 64 + 128, 64
     assert lib.tri_attn_bwd_noalloc(ctypes.byref(big)) == _lib.ESCRATCH
     assert lib.tri_attn_bwd_noalloc(None) == -1
+    # the combined backward checks the arguments of all three launches before the first one: a call without dK
+    # is refused as a whole, not after dQ and delta have been written (the pointers below are never followed)
+    part = _lib.TriAttnArgs()
+    part.struct_size = ctypes.sizeof(part)
+    part.dtype = 2
+    part.B, part.H, part.S, part.D = 1, 1, 256, 64
+    for name in ("q", "k", "v", "o", "lse", "d_o", "delta", "dq", "dv"):
+        setattr(part, name, 4096)
+    for name in ("q_stride", "k_stride", "v_stride", "o_stride", "do_stride", "dq_stride", "dk_stride", "dv_stride"):
+        getattr(part, name)[:] = [256 * 64, 256 * 64, 64, 1]
+    assert lib.tri_attn_bwd(ctypes.byref(part)) == -1  # dk missing
 
 
 def test_reference_value_errors():

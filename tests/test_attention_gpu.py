@@ -685,6 +685,123 @@ def test_classes_do_not_change_results(D, p, device):
             assert torch.equal(a, b_), (kind, name)
 
 
+@pytest.mark.parametrize("D", [64, 128])
+def test_dense_mask_gradient_behind_the_last_active_tile(D, device):
+    """A full-shape mask whose trailing key blocks are all -inf, with a gradient: the block classes let the kernels
+    stop streaming behind the last active tile, but the mask gradient written in place must still cover every tile
+    (zeros there). The buffer starts as NaN; results with and without classes are the same bits."""
+    import ctypes
+    from trident_amd import _lib, operation
+    lib = _lib.lib()
+    B, H, S = 1, 2, 512
+    dtype = torch.bfloat16
+    q, k, v, d_o = _gen((B, H, S, D), 91 + D, dtype)
+    mask = (0.5 * torch.randn(B, H, S, S, generator=torch.Generator().manual_seed(92))).to(dtype)
+    mask[..., 300:] = float("-inf")        # (key blocks from 320 on are -inf over every row)
+    mask[:, 1, 128:, 200:] = float("-inf")  # (and, for the lower rows of head 1, from 256 on)
+    tq, tk, tv, tdo, tm = [x.to(device) for x in (q, k, v, d_o, mask)]
+    scale = 1.0 / math.sqrt(D)
+    outs = []
+    for with_classes in (False, True):
+        o = torch.empty_like(tq)
+        lse = torch.empty(B, H, S, device=device)
+        delta = torch.empty_like(lse)
+        dq, dk, dv = [torch.full_like(tq, float("nan")) for _ in range(3)]
+        dmask = torch.full_like(tm, float("nan"))
+        args = operation._make_args(tq, tk, tv, o, lse, tm, 0.0, False, scale, 0, 0, tdo, dq, dk, dv, dmask, delta)
+        assert lib.tri_attn_uses_matrix_cores(ctypes.byref(args), 2) == 1
+        if with_classes:
+            classes = torch.empty(lib.tri_attn_mask_classes_size(ctypes.byref(args)), dtype=torch.uint8, device=device)
+            args.mask_classes = classes.data_ptr()
+            _lib.check(lib.tri_attn_classify_mask(ctypes.byref(args)))
+        _lib.check(lib.tri_attn_fwd(ctypes.byref(args)))
+        _lib.check(lib.tri_attn_bwd(ctypes.byref(args)))
+        torch.cuda.synchronize()
+        assert not torch.isnan(dmask.float()).any(), f"classes={with_classes}: part of the mask gradient was not written"
+        outs.append((o, dq, dk, dv, dmask))
+    for name, a, b_ in zip(("O", "dQ", "dK", "dV", "dMask"), *outs):
+        assert torch.equal(a, b_), name
+    o, dq, dk, dv, dmask = outs[1]
+    kw = dict(mask=mask, scale=scale)
+    o_ref, _ = parity.oracle_forward(q, k, v, **kw)
+    parity.close(o, o_ref, dtype, "O")
+    dq_r, dk_r, dv_r, dm_r, _ = parity.oracle_backward(q, k, v, d_o, want_dmask=True, o=o, **kw)
+    _, a_dq, a_dk, a_dv = parity.oracle_abs_sums(q, k, v, d_o, o=o, **kw)
+    parity.close(dq, dq_r, dtype, "dQ", a_dq)
+    parity.close(dk, dk_r, dtype, "dK", a_dk)
+    parity.close(dv, dv_r, dtype, "dV", a_dv)
+    parity.close(dmask, dm_r, dtype, "dMask")
+    # the same through the operator, which computes and passes the classes itself
+    _check(device, dtype, q, k, v, d_o, mask=mask, mask_grad=True, tag="operator dmask")
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_mask_written_between_two_calls(D, device):
+    """The operator keeps the block classes of a mask tensor between calls; writing to the tensor (version counter)
+    must bring fresh ones: the second mask opens keys the first one had masked out."""
+    B, H, S = 2, 2, 512
+    dtype = torch.bfloat16
+    q, k, v, _ = _gen((B, H, S, D), 93, dtype)
+    g = torch.Generator().manual_seed(94)
+    first = workloads.length_mask(B, S, g)[0]
+    second = torch.zeros_like(first)
+    second[:, :, :, :64] = float("-inf")
+    second[:, :, 256:, 200:330] = torch.randn(S - 256, 130, generator=g)
+    tq, tk, tv = [x.to(device) for x in (q, k, v)]
+    tm = first.to(device)
+    o1 = trident.function.scaled_dot_product_attention(tq, tk, tv, tm)
+    parity.close(o1, parity.oracle_forward(q, k, v, mask=first)[0], dtype, "first mask")
+    tm.copy_(second.to(device))
+    o2 = trident.function.scaled_dot_product_attention(tq, tk, tv, tm)
+    parity.close(o2, parity.oracle_forward(q, k, v, mask=second)[0], dtype, "second mask, same tensor")
+    # a write torch does not see needs forget_mask_classes() (or config.cache_mask_classes = False)
+    tm.data.copy_(first.to(device))
+    trident.operation.forget_mask_classes()
+    o3 = trident.function.scaled_dot_product_attention(tq, tk, tv, tm)
+    assert torch.equal(o3, o1)
+    trident.config.cache_mask_classes = False
+    try:
+        tm.data.copy_(second.to(device))
+        o4 = trident.function.scaled_dot_product_attention(tq, tk, tv, tm)
+        assert torch.equal(o4, o2)
+    finally:
+        trident.config.cache_mask_classes = True
+
+
+@pytest.mark.parametrize("dtype,S,D", [(torch.float32, 64, 32), (torch.bfloat16, 128, 32), (torch.bfloat16, 256, 64),
+                                       (torch.float32, 100, 128)])
+@pytest.mark.parametrize("scale", [-0.25, 0.0])
+def test_scales_that_are_not_positive(dtype, S, D, scale, device):
+    """softmax_scale <= 0 (function.attention accepts any value): the matrix-core kernels take row maxima before
+    scaling, so these problems run the element-wise kernels, which scale first."""
+    q, k, v, d_o = _gen((1, 2, S, D), 95, dtype)
+    for causal in (False, True):
+        _assert_kernel_family(q.to(device), None, 0.0, causal, scale, 0)
+        trident.config.reference_limits = False
+        try:
+            _check(device, dtype, q, k, v, d_o, is_causal=causal, scale=scale, tag=f"scale {scale}")
+        finally:
+            trident.config.reference_limits = True
+
+
+def test_config2_full_size(device):
+    """C2 at its full size (B=4, H=16: 256 items, one per compute unit through the persistent forward's item map):
+    two heads against the oracle, and V = 1 gives O = 1 everywhere."""
+    w = workloads.WORKLOADS["C2"]
+    q, k, v, _, _ = workloads.make_inputs(w)
+    tq, tk, tv = [x.to(device) for x in (q, k, v)]
+    out = trident.function.scaled_dot_product_attention(tq, tk, tv)
+    for (b, h) in [(0, 0), (3, 15), (2, 7)]:
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        o_ref, _ = parity.oracle_forward(q[sl], k[sl], v[sl])
+        parity.close(out[sl], o_ref, w.dtype, f"C2 head {b},{h} O")
+    o1 = trident.function.scaled_dot_product_attention(tq, tk, torch.ones_like(tv))
+    assert (o1.float() - 1).abs().max().item() <= 2.0**-10
+    perm = torch.randperm(w.H, generator=torch.Generator().manual_seed(2)).to(device)
+    o_p = trident.function.scaled_dot_product_attention(tq[:, perm], tk[:, perm], tv[:, perm])
+    assert torch.equal(o_p, out[:, perm])
+
+
 # ------------------------------------------------------------------ full-size properties
 def _abi_full(device, w, q, k, v, d_o, mask):
     """Forward + backward of a whole workload through the operator's two ABI wrappers; returns device tensors."""

@@ -4,7 +4,7 @@ import os
 import struct
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libtrident_attn.so")
+LIB_PATH = os.environ.get("TRIDENT_AMD_LIB") or os.path.join(_HERE, "libtrident_attn.so")  # (another build of the library)
 EALIGN = -8
 ENOFUSE = -9  # tri_attn_bwd_dq_delta: no fused kernel for this problem, nothing launched
 ABI_VERSION = 3

@@ -15,8 +15,15 @@ powers of two, boolean masks rejected with its error text, trident/operation/att
 the two that the kernels here do not need: any sequence length is accepted, and a boolean mask is taken the way
 torch.nn.functional.scaled_dot_product_attention takes it (True = the key takes part; it becomes an additive
 0 / -inf mask and has no gradient).
+
+``cache_mask_classes``: True keeps the classification of an additive mask's 64 x 64 blocks (all zero / all -inf / mixed,
+one pass over the mask) per mask tensor, so that the backward call and later calls with the same unmodified tensor reuse
+it. torch's version counter invalidates an entry; a write it does not see (``mask.data``, a raw pointer, a graph replay
+into the mask's memory) does not: set this to False then (every call classifies again), or call
+``trident_amd.operation.forget_mask_classes()`` after such a write.
 """
 use_autotune = True
 use_trace = False
 dropout_seed = None
 reference_limits = True
+cache_mask_classes = True

@@ -234,6 +234,12 @@ int tri_attn_bwd_dq_delta(const TriAttnArgs* args) {
 }
 
 int tri_attn_bwd(const TriAttnArgs* args) {
+    // (every argument is checked before the first launch: a call that fails leaves nothing half written)
+    {
+        KParams all;
+        const int bad = make_params(args, 2 | 4 | 8, &all);
+        if (bad) return bad;
+    }
     // Where the dQ kernel can compute delta on the way (it loads the dO rows anyway), the pre-pass is
     // dropped and dQ runs first: dK/dV reads the delta it stored.
     int rc = tri_attn_bwd_dq_delta(args);

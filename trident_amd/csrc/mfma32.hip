@@ -827,6 +827,7 @@ bool rows4(const void* ptr, const int64_t* s, int elem_bytes) {
 bool mfma32_supported(int which, int dtype, const KParams& p) {
     if (dtype < TRI_ATTN_F32 || dtype > TRI_ATTN_BF16) return false;
     if (p.D != 16 && p.D != 32 && p.D != 64 && p.D != 128) return false;
+    if (!(p.scale > 0.f)) return false;  // the forward takes row maxima before scaling
     const int eb = dtype == TRI_ATTN_F32 ? 4 : 2;
     // rows are read and written four elements at a time
     if (!rows4(p.q, p.qs, eb) || !rows4(p.k, p.ks, eb) || !rows4(p.v, p.vs, eb)) return false;

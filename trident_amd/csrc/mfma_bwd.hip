@@ -105,8 +105,12 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
             const TileClasses tc = tile_classes(p.mcls + b * p.mcs[0] + hd * p.mcs[1] + (q0 / 64) * p.mcs[2], 1, n_tiles,
                                                 kRows / 64, p.mcs[2], lane);
             zero_tiles = tc.zero;
-            n_tiles = tc.active ? 64 - __builtin_clzll(tc.active) : 1;
-            my_tiles = n_tiles;
+            // (a mask gradient written in place covers every tile: the tiles behind the last active one get their
+            // zeros from the loop; an accumulated one adds into a buffer the caller has zero-filled)
+            if (!DMASK || p.dmask_acc) {
+                n_tiles = tc.active ? 64 - __builtin_clzll(tc.active) : 1;
+                my_tiles = n_tiles;
+            }
         }
     }
     auto mask_is_zero = [&](int t) { return MASK != kNoMask && ((zero_tiles >> t) & 1) != 0; };
@@ -1300,8 +1304,8 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
     constexpr int KK = D / 16;
     constexpr int DB = D / 32;
     constexpr int DH = DB / 2;                               // column blocks a pair member accumulates
-    constexpr int kLoads = 3;                                // loads per wave and block
-    static_assert(kHalfBytes == NW * 1024, "one Q load and one dO load per wave and block");
+    constexpr int kLoads = 5;                                // loads per requesting wave and block
+    static_assert(kHalfBytes == NW * 1024, "two Q loads and two dO loads per requesting wave and block");
     constexpr int kAccSteps = 4 * DH;                        // MFMAs that add one block
     constexpr int kSteps = 2 * kAccSteps + 2 * KK;           // matrix phase
     constexpr int kRing = 4;
@@ -1339,34 +1343,37 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
 
     const int row_first = CAUSAL ? k0 : 0;          // first streamed row (block 0)
     const int n_blocks = (p.S - row_first) / kBR;   // >= 4, even
-    const uint32_t qoff = static_cast<uint32_t>(Tile::src_off(wave, lane, qrow_bytes));
-    const uint32_t goff = static_cast<uint32_t>(Tile::src_off(wave, lane, grow_bytes));
-    // Blocks are requested in order, one per phase (block ph + 4 in phase ph) after the first four: the
-    // source pointers and the ring slot advance with every call. Even waves fetch the 32 lse values of a
-    // block, odd waves its 32 delta values (lanes 32-63 repeat them).
-    int next_block = 0, next_slot = 0;
-    const char* next_q = qbase + row_first * qrow_bytes;
-    const char* next_g = gbase + row_first * grow_bytes;
-    const float* next_aux = ((wave & 1) ? delta_base : lse_base) + row_first;
-    const int aux_lds = 2 * kHalfBytes + ((wave & 1) ? 256 : 0);
-    auto issue_block = [&]() {  // this wave's share of the next block, if it exists
+    // A block is requested by the four waves of ONE member, the one that is in its vector phase when the request is
+    // due (member 0 the even blocks, member 1 the odd ones): a vector-memory instruction holds its wave until the
+    // memory pipeline has taken it, which the matrix phase cannot afford. Wave kb of the member fetches the 1 KiB
+    // pieces kb and kb + 4 of the Q rows and of the dO rows (rows 16 apart share the swizzle, so one per-lane offset
+    // serves both) and the block's 32 lse (kb even) or delta (kb odd) values; lanes 32-63 repeat those. The source
+    // pointers and the ring slot advance by two blocks per call.
+    const uint32_t qoff = static_cast<uint32_t>(Tile::src_off(kb, lane, qrow_bytes));
+    const uint32_t goff = static_cast<uint32_t>(Tile::src_off(kb, lane, grow_bytes));
+    int next_block = member, next_slot = member;
+    const char* next_q = qbase + (row_first + member * kBR) * qrow_bytes;
+    const char* next_g = gbase + (row_first + member * kBR) * grow_bytes;
+    const float* next_aux = ((kb & 1) ? delta_base : lse_base) + row_first + member * kBR;
+    const int aux_lds = 2 * kHalfBytes + ((kb & 1) ? 256 : 0);
+    auto issue_block = [&]() {  // this wave's share of its member's next block, if it exists
         if (next_block < n_blocks) {
             char* slot = smem + next_slot * kSlotBytes;
-            lds_direct_load16(next_q, qoff, slot + wave * 1024);
-            lds_direct_load16(next_g, goff, slot + kHalfBytes + wave * 1024);
+            lds_direct_load16(next_q, qoff, slot + kb * 1024);
+            lds_direct_load16(next_g, goff, slot + kHalfBytes + kb * 1024);
+            lds_direct_load16(next_q + 16 * qrow_bytes, qoff, slot + (kb + 4) * 1024);
+            lds_direct_load16(next_g + 16 * grow_bytes, goff, slot + kHalfBytes + (kb + 4) * 1024);
             lds_direct_load4(next_aux, (lane & 31) * 4, slot + aux_lds);
         }
-        ++next_block;
-        next_slot = next_slot == kSlots - 1 ? 0 : next_slot + 1;
-        next_q += kBR * qrow_bytes;
-        next_g += kBR * grow_bytes;
-        next_aux += kBR;
+        next_block += 2;
+        next_slot = next_slot >= kSlots - 2 ? next_slot + 2 - kSlots : next_slot + 2;
+        next_q += 2 * kBR * qrow_bytes;
+        next_g += 2 * kBR * grow_bytes;
+        next_aux += 2 * kBR;
     };
-    // before the barrier that ends phase ph: block ph+2 has landed, blocks ph+3 and ph+4 may be in flight
+    // before the barrier that ends vector phase ph of a member: its block ph+2 has landed, its block ph+4 may be in flight
     auto wait_blocks = [&](int ph) {
-        const int young = (ph + 3 < n_blocks ? 1 : 0) + (ph + 4 < n_blocks ? 1 : 0);
-        if (young == 2) TRI_WAIT_VMCNT(2 * kLoads);
-        else if (young == 1) TRI_WAIT_VMCNT(kLoads);
+        if (ph + 4 < n_blocks) TRI_WAIT_VMCNT(kLoads);
         else TRI_WAIT_VMCNT(0);
     };
 
@@ -1388,8 +1395,8 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
             lds_direct_load16(src, static_cast<uint32_t>(Tile::src_off(b16, lane, rb)), kv_lds + blk * 1024);
         }
     }
-#pragma unroll
-    for (int r = 0; r < 4; ++r) issue_block();
+    issue_block();  // blocks 0 and 2 (member 0), 1 and 3 (member 1)
+    issue_block();
 
     int row_off0 = Tile::off(l32, h);
     int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
@@ -1402,7 +1409,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
         tr_off0 = Tile::tr_off(0, 0, l);
         tr_off1 = Tile::tr_off(0, 1, l);
     };
-    TRI_WAIT_VMCNT(4 * kLoads);  // K and V have landed
+    TRI_WAIT_VMCNT(2 * kLoads);  // K and V have landed
     lds_barrier();
     u32x4 kf[KK], vf[KK];
 #pragma unroll
@@ -1422,7 +1429,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
         *reinterpret_cast<u32x4*>(my_xch + g * 1024) = cur_p[g];
         *reinterpret_cast<u32x4*>(my_xch + (2 + g) * 1024) = cur_s[g];
     }
-    TRI_WAIT_VMCNT(2 * kLoads);  // blocks 0 and 1 have landed
+    TRI_WAIT_VMCNT(kLoads);  // blocks 0 and 1 have landed
     lds_barrier();
 
     // whether this pair has anything in block r (under the causal mask: rows at or below its first key)
@@ -1587,27 +1594,17 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
         asm volatile("s_barrier" ::: "memory");  // (the reads above stay in flight)
         __builtin_amdgcn_sched_barrier(0);
     };
-    auto run_matrix_phase = [&](int ph, int r, int so) {
-        // this phase's loads first, while the ring's first fragments are still on their way (after the MFMAs
-        // they cost 1-1.6 % more cycles, between them 23 %)
+    auto run_matrix_phase = [&](int r, int so) {
         // (the last rounds have no own block to add and no block r + 2 to score: those steps are left out, except
         // with dropout, where the shorter instruction stream would cost registers the variant does not have)
-        issue_block();
-        __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_setprio(2);
         const int before = slot_step(so, -1);
         matrix_phase(Yes{}, r > 0 ? before : so, r < n_blocks ? so : before, slot_step(so, 2), DROPOUT || r < n_blocks,
                      DROPOUT || r + 2 < n_blocks);
         __builtin_amdgcn_s_setprio(0);
-        wait_blocks(ph);
         __builtin_amdgcn_sched_barrier(0);
         lds_barrier();
         __builtin_amdgcn_sched_barrier(0);
-    };
-    auto idle_phase = [&](int ph) {
-        issue_block();
-        wait_blocks(ph);
-        lds_barrier();
     };
 
     // before phase 0: S and dP of each member's first block (member 0: block 0, member 1: block 1)
@@ -1627,22 +1624,22 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
             const int r = 2 * t;
             vector_phase(r, so);
             close_vector_phase(2 * t, r, so);
-            run_matrix_phase(2 * t + 1, r, so);
+            run_matrix_phase(r, so);
             so = slot_step(so, 2);
         }
     } else {
         refresh_lane_offsets();
-        idle_phase(0);
+        lds_barrier();  // (phase 0: member 0 alone)
         int so = kSlotBytes;  // slot of block r
 #pragma unroll 1
         for (int t = 0; t < n_iter; ++t) {
             const int r = 2 * t + 1;
             vector_phase(r, so);
             close_vector_phase(2 * t + 1, r, so);
-            run_matrix_phase(2 * t + 2, r, so);
+            run_matrix_phase(r, so);
             so = slot_step(so, 2);
         }
-        idle_phase(2 * n_iter + 1);
+        lds_barrier();  // (the last phase: member 0 alone)
     }
 
     // every wave is out of the loop: the ring can serve as the waves' private transposition patches

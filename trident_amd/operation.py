@@ -85,8 +85,18 @@ def _make_args(query, key, value, output, log2sum, mask, dropout_p, is_causal, s
 
 # Classes of a mask's 64 x 64 blocks (tri_attn_classify_mask), kept per mask tensor: the forward call computes them, the
 # backward call and later calls with the same, unmodified tensor (other layers, other steps) find them here. An entry
-# dies with its tensor (weak reference) and is recomputed when the tensor was written to (its version counter moved).
+# dies with its tensor (weak reference) and is recomputed when the tensor was written to through torch (its version
+# counter moved), when another stream asks for it (no event orders the two), and it is neither made nor used while a
+# stream is being captured (the classification would be recorded, not run). A write that torch does not see (through
+# ``.data``, a raw pointer, a graph replay into the mask's memory) leaves stale classes behind, and the kernels skip
+# tiles on their word: such callers set ``config.cache_mask_classes = False`` (every call classifies the mask again)
+# or call ``forget_mask_classes()`` after the write.
 _MASK_CLASSES = {}
+
+
+def forget_mask_classes():
+    """Drops every cached block classification (after a write to a mask's memory that torch's version counter did not see)."""
+    _MASK_CLASSES.clear()
 
 
 def _mask_classes(mask: torch.Tensor, args):
@@ -98,9 +108,10 @@ def _mask_classes(mask: torch.Tensor, args):
     size = lib.tri_attn_mask_classes_size(ctypes.byref(args))
     if size <= 0:
         return None
+    use_cache = config.cache_mask_classes and not torch.cuda.is_current_stream_capturing()
     key = id(mask)
-    entry = _MASK_CLASSES.get(key)
-    signature = (mask._version, tuple(mask.shape), mask.stride(), mask.dtype, args.B, args.H, args.S, args.mask)
+    entry = _MASK_CLASSES.get(key) if use_cache else None
+    signature = (mask._version, tuple(mask.shape), mask.stride(), mask.dtype, args.B, args.H, args.S, args.mask, args.stream)
     if entry is not None and entry[0]() is mask and entry[1] == signature:
         classes = entry[2]
     else:
@@ -111,9 +122,10 @@ def _mask_classes(mask: torch.Tensor, args):
             args.mask_classes = None
             return None
         _lib.check(status)
-        if len(_MASK_CLASSES) >= 64:
-            _MASK_CLASSES.clear()
-        _MASK_CLASSES[key] = (weakref.ref(mask, lambda _r, k=key: _MASK_CLASSES.pop(k, None)), signature, classes)
+        if use_cache:
+            if len(_MASK_CLASSES) >= 64:
+                _MASK_CLASSES.clear()
+            _MASK_CLASSES[key] = (weakref.ref(mask, lambda _r, k=key: _MASK_CLASSES.pop(k, None)), signature, classes)
     args.mask_classes = classes.data_ptr()
     return classes
 
