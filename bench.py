@@ -376,7 +376,7 @@ def ceiling(dev):
 
     from trident_amd import _lib, workloads
 
-    lib = _lib.lib()
+    probe = _lib.probe_lib()
     peak = PEAK_TFLOPS["bf16"]
     res = {"peak_tflops": peak, "operands": "bf16 N(0,1) random (torch.randn, seed 1)"}
     torch.manual_seed(1)
@@ -398,12 +398,12 @@ def ceiling(dev):
 
     iters = 4000
     for mode, name in ((0, "mfma_registers"), (1, "mfma_lds_1_read_per_mfma"), (2, "mfma_lds_1_read_per_2_mfma")):
-        ms = timed(lambda: _lib.check(lib.tri_attn_probe_mfma(mode, cus, iters, operands.data_ptr(), out.data_ptr(),
+        ms = timed(lambda: _lib.check(probe.tri_probe_mfma(mode, cus, iters, operands.data_ptr(), out.data_ptr(),
                                                                torch.cuda.current_stream().cuda_stream)), 5)
         tf = cus * 8 * iters * 64 * 32768.0 / ms / 1e9
         res[name] = {"ms": round(ms, 3), "tflops": round(tf, 1), "frac_of_peak": round(tf / peak, 4),
                      "busy_x_clock_GHz": round(2.4 * tf / peak, 3)}
-    ms = timed(lambda: _lib.check(lib.tri_attn_probe_mfma(3, cus, iters // 4, operands.data_ptr(), out.data_ptr(),
+    ms = timed(lambda: _lib.check(probe.tri_probe_mfma(3, cus, iters // 4, operands.data_ptr(), out.data_ptr(),
                                                            torch.cuda.current_stream().cuda_stream)), 5)
     tf = cus * 8 * (iters // 4) * 64 * 4096.0 / ms / 1e9
     res["mfma_fp32_registers"] = {"ms": round(ms, 3), "tflops": round(tf, 1), "peak_tflops": PEAK_TFLOPS["fp32"],
@@ -415,7 +415,7 @@ def ceiling(dev):
         for valu, vname in ((0, "fma"), (1, "exp2"), (2, "fma_max_exp2")):
             row = {}
             for who, wname in ((1, "matrix_ms"), (2, "vector_ms"), (3, "both_ms"), (4, "same_wave_ms")):
-                row[wname] = round(timed(lambda: _lib.check(lib.tri_attn_probe_coexec(
+                row[wname] = round(timed(lambda: _lib.check(probe.tri_probe_coexec(
                     matrix, valu, who, cus, 2000, operands.data_ptr(), out.data_ptr(),
                     torch.cuda.current_stream().cuda_stream)), 3), 3)
             row["hidden_fraction_of_vector_work"] = round((row["matrix_ms"] + row["vector_ms"] - row["both_ms"]) / row["vector_ms"], 3)
@@ -452,6 +452,56 @@ def ceiling(dev):
     return res
 
 
+def sustained_clock(dev, seconds=1.5):
+    """The C3 step under sustained load with its seeded random operands and with all-zero operands (same launches, same
+    cycle counts): milliseconds per step and the shader clock and board power sampled meanwhile (torch.cuda.clock_rate /
+    power_draw, every 50 ms, second half of the run). The clock this load sustains depends on the operand bits, i.e. on
+    the power the matrix pipe draws: that, not the 2.4 GHz the published peak assumes, is what the kernels run at."""
+    import threading
+
+    import torch
+
+    from trident_amd import workloads
+
+    w = workloads.WORKLOADS["C3"]
+    res = {"workload": describe(w), "seconds_per_case": seconds}
+    for label in ("random_operands", "zero_operands", "random_operands_again"):
+        path = Path(w, dev)
+        if label == "zero_operands":
+            for t in (path.q, path.k, path.v, path.d_o):
+                t.zero_()
+        samples, stop = [], [False]
+
+        def sampler():
+            while not stop[0]:
+                try:
+                    samples.append((float(torch.cuda.clock_rate(dev)), float(torch.cuda.power_draw(dev))))
+                except Exception:  # (no management library on this box: the timing still stands)
+                    return
+                time.sleep(0.05)
+
+        th = threading.Thread(target=sampler)
+        th.start()
+        n, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(50):
+                for _, fn in path.kernels:
+                    fn()
+            torch.cuda.synchronize()
+            n += 50
+        dt = time.perf_counter() - t0
+        stop[0] = True
+        th.join()
+        tail = samples[len(samples) // 2:]
+        row = {"ms_per_step": round(dt / n * 1e3, 5), "tflops": round(w.flops(True) / (dt / n) / 1e12, 1), "samples": len(tail)}
+        if tail:
+            row["clock_mhz"] = round(sum(x[0] for x in tail) / len(tail))
+            row["power_draw_raw"] = round(sum(x[1] for x in tail) / len(tail))
+        res[label] = row
+        del path
+    return res
+
+
 def describe(w):
     extra = "causal" if w.is_causal else ("additive fp32 mask [B,1,S,S]" if w.masked else "plain")
     if w.dropout_p:
@@ -476,6 +526,9 @@ def main():
     ap.add_argument("--ceiling", action="store_true",
                     help="instead of the benchmark: print one JSON line with the MFMA ceiling of this box (random-operand "
                          "MFMA loops, a bf16 GEMM, the C3 kernels)")
+    ap.add_argument("--sustained-clock", action="store_true",
+                    help="instead of the benchmark: one JSON line with the C3 step under sustained load, its seeded random "
+                         "operands against all-zero operands, and the shader clock sampled meanwhile")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (known HBM traffic) so that rocprofv3 FETCH_SIZE / "
@@ -495,6 +548,9 @@ def main():
     w = {**workloads.WORKLOADS, **workloads.EXTRA_WORKLOADS}[a.workload]
     if a.ceiling:
         print(json.dumps({"ceiling": ceiling(dev)}), flush=True)
+        return
+    if a.sustained_clock:
+        print(json.dumps({"sustained_clock": sustained_clock(dev)}), flush=True)
         return
     if a.sibling_ops:
         print(json.dumps({"sibling_ops": sibling_ops(dev)}), flush=True)

@@ -25,6 +25,17 @@ def test_library_exports_every_declared_symbol():
     assert lib.tri_attn_version() == _lib.ABI_VERSION
 
 
+def test_probe_library_exports_its_header():
+    """The calibration kernels live in a library and header of their own, outside the operator's boundary."""
+    text = open(os.path.join(ROOT, "include", "tri_probe.h")).read()
+    declared = set(re.findall(r"\b(tri_probe_\w+)\s*\(", text))
+    assert declared == set(_lib.PROBE_EXPORTS)
+    assert not re.search(r"tri_\w*probe", open(HEADER).read())
+    lib = _lib.probe_lib()
+    for name in declared:
+        assert hasattr(lib, name)
+
+
 def test_struct_layout_matches_header(tmp_path):
     src = tmp_path / "sz.c"
     src.write_text(

@@ -99,8 +99,6 @@ EXPORTS = (
     "tri_attn_uses_matrix_cores",
     "tri_attn_classify_mask",
     "tri_attn_mask_classes_size",
-    "tri_attn_probe_mfma",
-    "tri_attn_probe_coexec",
 )
 
 _lib = None
@@ -140,16 +138,32 @@ def lib():
             fn = getattr(cdll, name)  # AttributeError if a declared symbol is not exported
             fn.restype = ctypes.c_int
             fn.argtypes = [ctypes.POINTER(TriRowArgs)]
-        cdll.tri_attn_probe_mfma.restype = ctypes.c_int
-        cdll.tri_attn_probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
-                                             ctypes.c_void_p, ctypes.c_void_p]
-        cdll.tri_attn_probe_coexec.restype = ctypes.c_int
-        cdll.tri_attn_probe_coexec.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-                                               ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
         if cdll.tri_attn_version() != ABI_VERSION:
             raise RuntimeError("libtrident_attn.so ABI version mismatch: rebuild it")
         _lib = cdll
     return _lib
+
+
+PROBE_LIB_PATH = os.path.join(_HERE, "libtri_probe.so")
+PROBE_EXPORTS = ("tri_probe_mfma", "tri_probe_coexec")
+_probe = None
+
+
+def probe_lib():
+    """The calibration kernels of include/tri_probe.h (a library of their own; only bench.py --ceiling loads it)."""
+    global _probe
+    if _probe is None:
+        if not os.path.exists(PROBE_LIB_PATH):
+            raise RuntimeError(f"{PROBE_LIB_PATH} is missing: build it with `python -m trident_amd.build`")
+        cdll = ctypes.CDLL(PROBE_LIB_PATH)
+        cdll.tri_probe_mfma.restype = ctypes.c_int
+        cdll.tri_probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
+                                        ctypes.c_void_p]
+        cdll.tri_probe_coexec.restype = ctypes.c_int
+        cdll.tri_probe_coexec.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                          ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+        _probe = cdll
+    return _probe
 
 
 def check(status):

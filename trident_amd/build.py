@@ -18,6 +18,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 OUT = os.path.join(HERE, "libtrident_attn.so")
+PROBE_SRC = os.path.join(HERE, "probe", "probe.hip")   # calibration kernels: a library of their own (include/tri_probe.h)
+PROBE_OUT = os.path.join(HERE, "libtri_probe.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -151,14 +153,16 @@ def check_baseline_kernels(resources):
 def build(verbose=True, resources=False):
     os.makedirs(OBJ_DIR, exist_ok=True)
     sources = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
-    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
-        results = list(pool.map(_compile, sources))
+    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(sources) + 1)) as pool:
+        results = list(pool.map(_compile, sources + [PROBE_SRC]))
+    probe_obj = results.pop()[0]
     objs = [o for o, _ in results]
     usage = {}
     for _, r in results:
         usage.update(r)
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", OUT, *objs]
     subprocess.check_call(cmd)
+    subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", PROBE_OUT, probe_obj])
     if resources:
         print(resource_table(usage))
     check_baseline_kernels(usage)

@@ -1,4 +1,6 @@
 // Which calls the matrix-core kernels take, and the delta pre-pass.
+#include <atomic>
+
 #include "launch.hpp"
 #include "mfma_common.hpp"
 
@@ -147,15 +149,15 @@ bool mfma_dq_fuses_delta(const KParams& p) {
 }
 
 int persistent_grid(int items) {
-    static int cus[64] = {};  // per device ordinal; 0 = not asked yet
+    static std::atomic<int> cus[64];  // per device ordinal; 0 = not asked yet (every thread would store the same value)
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return items;
-    if (cus[dev] == 0) {
-        int n = 0;
+    int n = cus[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
         if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return items;
-        cus[dev] = n;
+        cus[dev].store(n, std::memory_order_relaxed);
     }
-    return items < cus[dev] ? items : cus[dev];
+    return items < n ? items : n;
 }
 
 int launch_delta(int dtype, const KParams& p, hipStream_t stream) {

@@ -1,9 +1,10 @@
-// Calibration kernels: what the matrix pipe of this GPU sustains on random operands, alone and with its A
-// operands streamed from LDS. They have no counterpart in the reference; bench.py --ceiling times them next
+// Calibration kernels (libtri_probe.so, include/tri_probe.h; not part of the operator's library): what the matrix pipe
+// of this GPU sustains on random operands, alone and with its A operands streamed from LDS. They have no counterpart in
+// the reference; bench.py --ceiling times them next
 // to a large bf16 GEMM and the attention kernels, so that an attention kernel's distance from the published
 // MFMA peak can be split into "cycles not spent in MFMAs" and "clock below 2.4 GHz under this load".
-#include "launch.hpp"
 #include "mfma_common.hpp"
+#include "tri_probe.h"
 
 namespace tri {
 namespace {
@@ -158,7 +159,7 @@ __global__ __launch_bounds__(kProbeThreads) void coexec_kernel(const u32x4* __re
 
 using namespace tri;
 
-extern "C" int tri_attn_probe_coexec(int matrix, int valu, int who, int workgroups, int iters, const void* operands,
+extern "C" int tri_probe_coexec(int matrix, int valu, int who, int workgroups, int iters, const void* operands,
                                      float* out, void* stream) {
     if (operands == nullptr || out == nullptr) return TRI_ATTN_ENULL;
     if (workgroups <= 0 || iters <= 0 || matrix < 0 || matrix > 1 || valu < 0 || valu > 2 || who < 1 || who > 4) return TRI_ATTN_ESHAPE;
@@ -175,7 +176,7 @@ extern "C" int tri_attn_probe_coexec(int matrix, int valu, int who, int workgrou
     return static_cast<int>(hipGetLastError());
 }
 
-extern "C" int tri_attn_probe_mfma(int mode, int workgroups, int iters, const void* operands, float* out, void* stream) {
+extern "C" int tri_probe_mfma(int mode, int workgroups, int iters, const void* operands, float* out, void* stream) {
     if (operands == nullptr || out == nullptr) return TRI_ATTN_ENULL;
     if (workgroups <= 0 || iters <= 0 || mode < 0 || mode > 3) return TRI_ATTN_ESHAPE;
     const dim3 grid(workgroups), block(kProbeThreads);
