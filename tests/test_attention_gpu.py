@@ -784,6 +784,20 @@ def test_scales_that_are_not_positive(dtype, S, D, scale, device):
             trident.config.reference_limits = True
 
 
+@pytest.mark.parametrize("mask_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mask_grad", [False, True])
+def test_mask_with_dropout_at_the_large_head(mask_dtype, mask_grad, device):
+    """D = 128 with a mask and dropout together (and a mask gradient on top): the variants that do not fit the 8-wave
+    kernels' registers take a smaller fragment ring (forward) or 128-row workgroups (dQ); no kernel of the library uses
+    scratch memory."""
+    B, H, S, D = 1, 2, 512, 128
+    q, k, v, d_o = _gen((B, H, S, D), 96, torch.bfloat16)
+    mask = (0.5 * torch.randn(B, H, S, S, generator=torch.Generator().manual_seed(97))).to(mask_dtype)
+    _assert_kernel_family(q.to(device), mask.to(device), 0.2, False, 1.0 / math.sqrt(D), 1)
+    _check(device, torch.bfloat16, q, k, v, d_o, mask=mask, dropout_p=0.2, mask_grad=mask_grad, seed=98,
+           tag=f"mask {mask_dtype} + dropout, D=128")
+
+
 def test_config2_full_size(device):
     """C2 at its full size (B=4, H=16: 256 items, one per compute unit through the persistent forward's item map):
     two heads against the oracle, and V = 1 gives O = 1 everywhere."""

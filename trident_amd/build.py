@@ -3,9 +3,10 @@
     python -m trident_amd.build               # compile every csrc/*.hip and link
     python -m trident_amd.build --resources   # also print the per-kernel register / LDS / scratch table
 
-Every build reads the compiler's kernel-resource-usage remarks and FAILS when a kernel that one of the five
-benchmark configurations launches uses scratch memory (spilled vector registers): a scratch reload is a
-vector-memory load, and the kernels' hand-counted vmcnt waits would then drain the tile prefetch on every reload.
+Every build reads the compiler's kernel-resource-usage remarks and FAILS when any kernel of the library uses scratch
+memory (spilled vector registers): a scratch reload is a vector-memory load, and the kernels' hand-counted vmcnt waits
+would then drain the tile prefetch on every reload. It also fails when a kernel of the five benchmark configurations is
+missing from the build.
 """
 import concurrent.futures
 import glob
@@ -144,10 +145,10 @@ def check_baseline_kernels(resources):
     missing = [k for k in BASELINE_KERNELS if k not in found]
     if missing:
         raise RuntimeError("kernels of the benchmark configurations not found in the build: " + ", ".join(missing))
-    bad = [f"{k} ({BASELINE_KERNELS[k]}): {found[k].get('scratch', 0)} bytes of scratch per lane"
-           for k in BASELINE_KERNELS if found[k].get("scratch", 0) > 0]
+    bad = [f"{k}{' (' + BASELINE_KERNELS[k] + ')' if k in BASELINE_KERNELS else ''}: {r.get('scratch', 0)} bytes of scratch per lane"
+           for k, r in sorted(found.items()) if r.get("scratch", 0) > 0]
     if bad:
-        raise RuntimeError("benchmark kernels spill vector registers to scratch:\n  " + "\n  ".join(bad))
+        raise RuntimeError("kernels spill vector registers to scratch:\n  " + "\n  ".join(bad))
 
 
 def build(verbose=True, resources=False):
@@ -167,7 +168,7 @@ def build(verbose=True, resources=False):
         print(resource_table(usage))
     check_baseline_kernels(usage)
     if verbose:
-        print(f"built {OUT} from {len(sources)} sources; {len(usage)} kernels, none of the benchmark kernels uses scratch")
+        print(f"built {OUT} from {len(sources)} sources; {len(usage)} kernels, none uses scratch")
     return OUT
 
 

@@ -1665,15 +1665,23 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
 template <typename T, int D, int NW, bool CAUSAL, int MASK>
 int launch_dq_waves(const KParams& p, hipStream_t stream) {
     const dim3 grid(p.B * p.H * (p.S / (32 * NW))), block(64 * NW);
-    if constexpr (MASK != kNoMask) {
-        if (p.dmask != nullptr) {
-            if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dq_kernel<T, D, NW, CAUSAL, MASK, true, false, true>), grid, block, 0, stream, p);
-            else hipLaunchKernelGGL((mfma_dq_kernel<T, D, NW, CAUSAL, MASK, false, false, true>), grid, block, 0, stream, p);
-            return static_cast<int>(hipGetLastError());
+    if constexpr (NW == 8 && D == 128 && MASK != kNoMask) {
+        // with a mask gradient or dropout on top of a mask the 8-wave kernel does not fit its registers at D = 128 and
+        // would spill to scratch memory (whose reloads are vector-memory loads that drain the tile prefetch): those
+        // problems take 128-row workgroups, which fit
+        if (p.dmask != nullptr || p.thr8 > 0) return launch_dq_waves<T, D, 4, CAUSAL, MASK>(p, stream);
+        hipLaunchKernelGGL((mfma_dq_kernel<T, D, NW, CAUSAL, MASK, false>), grid, block, 0, stream, p);
+    } else {
+        if constexpr (MASK != kNoMask) {
+            if (p.dmask != nullptr) {
+                if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dq_kernel<T, D, NW, CAUSAL, MASK, true, false, true>), grid, block, 0, stream, p);
+                else hipLaunchKernelGGL((mfma_dq_kernel<T, D, NW, CAUSAL, MASK, false, false, true>), grid, block, 0, stream, p);
+                return static_cast<int>(hipGetLastError());
+            }
         }
+        if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dq_kernel<T, D, NW, CAUSAL, MASK, true>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((mfma_dq_kernel<T, D, NW, CAUSAL, MASK, false>), grid, block, 0, stream, p);
     }
-    if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dq_kernel<T, D, NW, CAUSAL, MASK, true>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((mfma_dq_kernel<T, D, NW, CAUSAL, MASK, false>), grid, block, 0, stream, p);
     return static_cast<int>(hipGetLastError());
 }
 

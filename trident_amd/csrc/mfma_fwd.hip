@@ -47,12 +47,13 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     constexpr int DB = D / 32;  // 32-row blocks of O^T
     constexpr int kSteps = 2 * KK;    // MFMAs of S^T per tile
     constexpr int kPvSteps = 4 * DB;  // MFMAs of O^T per tile
-    constexpr int kRing = 6;          // operand fragments in flight
+    // operand fragments in flight (a mask and dropout together at D = 128 leave room for four only)
+    constexpr int kRing = (D == 128 && MASK != kNoMask && DROPOUT) ? 4 : 6;
     // A mask block of a wave (32 rows x 64 keys) goes through a private LDS region (8 KiB for an fp32 mask, 4 KiB
     // for one of the operand type) when it fits (D = 64): lanes own rows, so direct loads would touch 32 cache
     // lines per instruction, while LDS-direct loads fetch whole rows (256 or 128 bytes) and the swizzled tile is
     // read back 16 or 8 bytes at a time. The region has the geometry of a 32-row SwzTile<128> / SwzTile<64>.
-    constexpr bool kMaskViaLds = MASK != kNoMask && (D == 64 || (MASK == kMaskT && NW == 8));  // (D = 128: 4 KiB regions fit, 8 KiB ones do not)
+    constexpr bool kMaskViaLds = MASK != kNoMask && (D == 64 || (MASK == kMaskT && NW == 8 && !DROPOUT));  // (D = 128: 4 KiB regions fit, 8 KiB ones do not; with dropout the registers for the staged values are not there)
     constexpr int kMaskElt = MASK == kMaskF32 ? 4 : 2;
     using MaskTile = std::conditional_t<MASK == kMaskF32, SwzTile<128>, SwzTile<64>>;
     constexpr int kMaskBytes = 32 * MaskTile::kRowBytes;
@@ -437,7 +438,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
                 if (ks < 2 && issued) issue_slice(j + dist, 2 + ks);
                 if (ks < 2) {
 #pragma unroll
-                    for (int r = 3 * ks; r < 3 * ks + 3; ++r) ring[r] = frag(Yes{}, j, r);
+                    for (int r = kRing / 2 * ks; r < kRing / 2 * (ks + 1); ++r) ring[r] = frag(Yes{}, j, r);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -476,7 +477,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
                 for (int ks = 0; ks < 4; ++ks) pb[ks] = pack8<T>(&x[8 * ks]);
             }
         }
-        static_assert(kRing == 6, "the softmax phase requests fragments 0..5");
+        static_assert(kRing % 2 == 0, "the softmax phase requests the first fragments in two halves");
 
         const bool with_s = j + 1 < my_tiles;
         // tile j+dist-1 has landed (the next mask block and the newest tile may still be in flight);
