@@ -1559,8 +1559,22 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
             const int rb = row_first + r * kBR;
             softmax_backward(CAUSAL && r == kb, rb, so);
         } else {
+            // (the zeros are made inside this branch, where the compiler cannot lift them in front of the test above:
+            // lifted, they are sixteen moves in every phase of the loop. The one variant that has no two registers to
+            // spare for that keeps the plain assignment.)
+            constexpr bool kPlainZeros = std::is_same<T, f16_t>::value && CAUSAL && !DROPOUT;
 #pragma unroll
-            for (int g = 0; g < 2; ++g) cur_p[g] = cur_s[g] = u32x4{0, 0, 0, 0};
+            for (int g = 0; g < 2; ++g) {
+                if constexpr (kPlainZeros) {
+                    cur_p[g] = cur_s[g] = u32x4{0, 0, 0, 0};
+                } else {
+                    uint32_t z[8];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) asm volatile("v_mov_b32 %0, 0" : "=v"(z[i]));
+                    cur_p[g] = u32x4{z[0], z[1], z[2], z[3]};
+                    cur_s[g] = u32x4{z[4], z[5], z[6], z[7]};
+                }
+            }
         }
     };
     // the second half of a vector phase in global phase ph, for a member whose block is r: publish, fetch
