@@ -171,7 +171,10 @@ int tri_attn_bwd_noalloc(const TriAttnArgs* args);
  * tri_attn_mask_classes_size(args) bytes). It has no counterpart in the reference, whose kernel adds every mask
  * tile as it comes (trident/kernel/attention.py:135-138). With the classes at hand the kernels skip key tiles
  * that are masked out altogether and do not read mask tiles that are all zero (a key-padding or length mask is
- * made of such tiles but for one column of blocks); results are unchanged. Reads mask; writes mask_classes.
+ * made of such tiles but for one column of blocks). A tile whose mask is all zero then takes the arithmetic of a tile
+ * without a mask (the scale folded into one fused multiply-add per score instead of a product, a sum and a
+ * difference): results agree with those computed without classes to the last fp32 rounding of a score's exponent, i.e.
+ * to within an ulp of the 16-bit outputs, not bit for bit. Reads mask; writes mask_classes.
  * Returns TRI_ATTN_ENOFUSE (nothing launched) where the classes would not be used: S not a multiple of 128. */
 int tri_attn_classify_mask(const TriAttnArgs* args);
 /* Bytes of mask_classes for these arguments (MB * MH * RB * S/64), 0 where tri_attn_classify_mask does not apply, or a

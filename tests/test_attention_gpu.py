@@ -651,7 +651,7 @@ def test_mask_block_classes(mshape, mask_dtype, device):
 
 @pytest.mark.parametrize("D,p", [(64, 0.0), (128, 0.0), (64, 0.3)])
 def test_classes_do_not_change_results(D, p, device):
-    """The same calls with and without mask_classes give the same bits: skipped tiles only ever added zeros."""
+    """The same calls with and without mask_classes give the same results: skipped tiles only ever added zeros."""
     import ctypes
     from trident_amd import _lib, operation
     lib = _lib.lib()
@@ -680,9 +680,18 @@ def test_classes_do_not_change_results(D, p, device):
             _lib.check(lib.tri_attn_bwd(ctypes.byref(args)))
             torch.cuda.synchronize()
             outs.append((o, lse, dq, dk, dv))
+        # a tile whose mask is all zero takes the arithmetic of a tile without a mask (one fused multiply-add per score
+        # instead of product, sum and difference): the same results up to that fp32 rounding of the exponents
         for name, a, b_ in zip(("O", "LSE", "dQ", "dK", "dV"), *outs):
             assert not torch.isnan(a.float()).any(), (kind, name)
-            assert torch.equal(a, b_), (kind, name)
+            a32, b32 = a.float(), b_.float()
+            if name == "LSE":
+                assert (a32 - b32).abs().max().item() <= 2e-5, (kind, name)
+            else:
+                # within a bf16 ulp of the tensor's scale (sums with cancellation move by an ulp of their terms), and
+                # nearly all elements equal
+                assert (a32 - b32).abs().max().item() <= 2.0**-8 * a32.abs().max().item(), (kind, name)
+                assert (a32 != b32).float().mean().item() < 0.2, (kind, name)
 
 
 @pytest.mark.parametrize("D", [64, 128])

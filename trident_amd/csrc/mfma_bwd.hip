@@ -183,10 +183,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
         float mk2[kMaskViaLds ? 32 : 1];
         if constexpr (kMaskViaLds) {
             // (a mask excludes the causal variant, so every wave works on every tile)
-            if (mask_is_zero(j)) {
-#pragma unroll
-                for (int i = 0; i < 32; ++i) mk2[i] = 0.f;
-            } else {
+            if (!mask_is_zero(j)) {  // (a tile whose mask is all zero takes the arithmetic of a tile without a mask)
 #pragma unroll
                 for (int g = 0; g < 8; ++g) {  // keys 8 g + 4 h .. + 3 of this lane's row
                     if constexpr (MASK == kMaskF32) {
@@ -212,9 +209,13 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
             float mk[MASK != kNoMask ? 16 : 1];
+            // (at D = 128 the registers do not hold a second form of the arithmetic: a tile whose mask is all zero adds zeros)
+            const bool masked = MASK != kNoMask && (D == 128 || !mask_is_zero(j));
             if constexpr (kMaskViaLds) {
+                if (masked) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) mk[i] = mk2[16 * kb + i];
+                    for (int i = 0; i < 16; ++i) mk[i] = mk2[16 * kb + i];
+                }
             } else if constexpr (MASK != kNoMask) {
                 if (mask_is_zero(j)) {
 #pragma unroll
@@ -254,12 +255,12 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
                 for (int i = 0; i < 16; ++i) st[i] = t0 + 32 * kb + c_row(i, h) < p.S ? st[i] : -INFINITY;
             }
             float ds[16];
+            if (masked) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                float pr;
-                if constexpr (MASK != kNoMask) pr = fast_exp2(fmaf(mk[i], kLog2e, st[i] * c) - lse);
-                else pr = fast_exp2(fmaf(st[i], c, -lse));
-                ds[i] = pr;
+                for (int i = 0; i < 16; ++i) ds[i] = fast_exp2(fmaf(mk[i], kLog2e, st[i] * c) - lse);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) ds[i] = fast_exp2(fmaf(st[i], c, -lse));
             }
             if constexpr (DROPOUT) {
                 const Philox4 mine = dropout_block(p, bh, qrow >> 2, (t0 + 32 * kb + 8 * (lane & 3) + 4 * h) >> 2);
@@ -743,10 +744,7 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
         float mk2[kMaskViaLds ? 32 : 1];
         if constexpr (kMaskViaLds) {
             // (a mask excludes the causal variant, so every wave works on every tile)
-            if (mask_is_zero(j)) {
-#pragma unroll
-                for (int i = 0; i < 32; ++i) mk2[i] = 0.f;
-            } else {
+            if (!mask_is_zero(j)) {  // (a tile whose mask is all zero takes the arithmetic of a tile without a mask)
 #pragma unroll
                 for (int i = 0; i < 32; ++i) {  // row 32 (i / 16) + c_row(i % 16, h), this lane's key
                     const int row = 32 * (i >> 4) + c_row(i & 15, h);
@@ -773,14 +771,14 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
             const int rb = r0 + 32 * qb;
             if (CAUSAL && rb + 31 < wkey0) continue;  // whole block above the wave's keys
             float mk[MASK != kNoMask ? 16 : 1];
+            const bool masked = MASK != kNoMask && !mask_is_zero(j);
             if constexpr (kMaskViaLds) {
+                if (masked) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) mk[i] = qb ? mk2[16 + i] : mk2[i];  // static indices keep it in registers
+                    for (int i = 0; i < 16; ++i) mk[i] = qb ? mk2[16 + i] : mk2[i];  // static indices keep it in registers
+                }
             } else if constexpr (MASK != kNoMask) {
-                if (mask_is_zero(j)) {
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) mk[i] = 0.f;
-                } else {
+                if (masked) {
                     const int64_t mbase = b * p.ms[0] + hd * p.ms[1] + key;
 #pragma unroll
                     for (int i = 0; i < 16; ++i)
@@ -814,11 +812,27 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
             u32x4 pb[2], sb[2];
             {
                 float pr[16], ds[16];
+                // the probabilities first: with the mask's values, or as in a tile without a mask where they are all zero
+                float pexp[16];
+                if (masked) {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + 32 * qb + 8 * g + 4 * h);
+#pragma unroll
+                        for (int bb = 0; bb < 4; ++bb) pexp[4 * g + bb] = fast_exp2(fmaf(mk[4 * g + bb], kLog2e, s[4 * g + bb] * c) - l4[bb]);
+                    }
+                } else {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + 32 * qb + 8 * g + 4 * h);
+#pragma unroll
+                        for (int bb = 0; bb < 4; ++bb) pexp[4 * g + bb] = fast_exp2(fmaf(s[4 * g + bb], c, -l4[bb]));
+                    }
+                }
                 Philox4 mine;  // the block of rows rb + 8 (lane % 4) + 4 h .. +3: this lane's share of the quad's four
                 if constexpr (DROPOUT) mine = dropout_block(p, bh, (rb + 8 * (lane & 3) + 4 * h) >> 2, key >> 2);
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + 32 * qb + 8 * g + 4 * h);
                     const f32x4 d4 = *reinterpret_cast<const f32x4*>(sDelta + 32 * qb + 8 * g + 4 * h);
                     uint32_t dw[4];
                     if constexpr (DROPOUT) {
@@ -829,9 +843,7 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
 #pragma unroll
                     for (int bb = 0; bb < 4; ++bb) {
                         const int i = 4 * g + bb;
-                        float pv;
-                        if constexpr (MASK != kNoMask) pv = fast_exp2(fmaf(mk[i], kLog2e, s[i] * c) - l4[bb]);
-                        else pv = fast_exp2(fmaf(s[i], c, -l4[bb]));
+                        const float pv = pexp[i];
                         float dpv = dp[i];
                         if constexpr (DROPOUT) {
                             const bool keep = static_cast<int>(dw[bb]) >= p.thr8;

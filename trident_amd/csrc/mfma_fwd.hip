@@ -209,11 +209,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     // additive mask values of this lane's row for tile t, straight from memory
     auto load_mask = [&](int t) {
         if constexpr (MASK != kNoMask && !kMaskViaLds) {
-            if (mask_is_zero(t)) {
-#pragma unroll
-                for (int e = 0; e < 32; ++e) mk[e] = 0.f;
-                return;
-            }
+            if (mask_is_zero(t)) return;  // (the tile then takes the arithmetic of a tile without a mask: mk is not read)
             const int64_t mrow = b * p.ms[0] + hd * p.ms[1] + static_cast<int64_t>(qrow) * p.ms[2] + t * kBN;
 #pragma unroll
             for (int g = 0; g < 8; ++g) {
@@ -234,10 +230,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
         if constexpr (kMaskViaLds) {
             // block t was requested a matrix phase ago and only the newest tile load may be younger
             // (block 0 precedes tile 0, which has landed)
-            if (mask_is_zero(t)) {
-#pragma unroll
-                for (int e = 0; e < 32; ++e) mk[e] = 0.f;
-            } else {
+            if (!mask_is_zero(t)) {
                 if (!first) wait_loads(false, tile_in_flight);
 #pragma unroll
                 for (int g = 0; g < 8; ++g) {  // keys 32 (g / 4) + 8 (g % 4) + 4 h .. + 3 of this lane's row
@@ -272,8 +265,9 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     // the matrix phase, one or two per MFMA of the first key block's P V steps: that phase has issue slots
     // to spare, the softmax phase is the one the partner waits for.
     constexpr bool kDefer = !DROPOUT;
-    float xd[16];        // deferred exponents (already scaled, masked) and then probabilities
+    float xd[16];        // deferred exponents and then probabilities
     float m_def = 0.f;   // the reference exponent they are taken against
+    float c_def = c;     // the factor they are still to be multiplied by (1 where the mask has been added: scaled already)
     const uint32_t one2 = Mma<T>::pack2(1.f, 1.f);
     const u32x4 ones = {one2, one2, one2, one2};
     f32x16 lacc = zero16();
@@ -319,7 +313,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
                         if (e * ne / 8 == ls) {
                             float& v = xd[8 * (g - 2) + e];
                             if constexpr (MASK == kNoMask) v = fast_exp2(fmaf(v, c, -m_def));
-                            else v = fast_exp2(v - m_def);
+                            else v = fast_exp2(fmaf(v, c_def, -m_def));
                         }
                     if (ls == pack_step) pb[g] = pack8<T>(&xd[8 * (g - 2)]);
                 }
@@ -376,10 +370,15 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
                 x[i] = sc[0][i];
                 x[16 + i] = sc[1][i];
             }
-            // scores in the log2 domain; without a mask the scale is folded into the exponent
+            // scores in the log2 domain; without a mask - and in a tile whose mask is all zero - the scale is folded into
+            // the exponent's multiply-add (cc: the factor still to apply)
+            float cc = c;
             if constexpr (MASK != kNoMask) {
+                if (!mask_is_zero(j)) {
 #pragma unroll
-                for (int e = 0; e < 32; ++e) x[e] = fmaf(mk[e], kLog2e, x[e] * c);
+                    for (int e = 0; e < 32; ++e) x[e] = fmaf(mk[e], kLog2e, x[e] * c);
+                    cc = 1.f;
+                }
             }
             if (CAUSAL && t0 + kBN - 1 > wrow0) {
 #pragma unroll
@@ -402,7 +401,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
                 mx1 = fmaxf(mx1, x[16 + e]);
             }
             mx = max_xor32(fmaxf(mx, mx1));
-            if constexpr (MASK == kNoMask) mx *= c;
+            mx *= cc;
             // Lazy rescaling: m is the reference exponent of l and of the O accumulators, not
             // necessarily the running maximum. It is only moved (and O rescaled) when some row of
             // the wave outgrew it by more than 2^kTau; until then probabilities may exceed 1 by
@@ -432,7 +431,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
 #pragma unroll
                 for (int e = 8 * ks; e < 8 * ks + 8; ++e) {
                     if constexpr (MASK == kNoMask) x[e] = fast_exp2(fmaf(x[e], c, -m_use));
-                    else x[e] = fast_exp2(x[e] - m_use);
+                    else x[e] = fast_exp2(fmaf(x[e], cc, -m_use));
                 }
                 if constexpr (!DROPOUT) pb[ks] = pack8<T>(&x[8 * ks]);
                 if (ks < 2 && issued) issue_slice(j + dist, 2 + ks);
@@ -446,6 +445,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) xd[e] = x[16 + e];
                 m_def = m_use;
+                c_def = cc;
             }
             if constexpr (DROPOUT) {
                 // row sum before dropping, in fp32: four interleaved partial sums (a dependent add waits
