@@ -107,7 +107,13 @@ __device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32); }
 // the swap leaves {x[l % 32], x[l % 32 + 32]} in the two registers of every lane. The instruction
 // needs two wait states after a vector write of its operands.
 __device__ __forceinline__ void swap32(float& a, float& b) { asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
-__device__ __forceinline__ float max_xor32(float x) { float a = x, b = x; swap32(a, b); return fmaxf(a, b); }
+// v_max3_f32 as it stands (scores are never signalling NaNs; fmaxf would canonicalise its operands first)
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+__device__ __forceinline__ float max_xor32(float x) { float a = x, b = x; swap32(a, b); return max3(a, b, b); }
 __device__ __forceinline__ float sum_xor32(float x) { float a = x, b = x; swap32(a, b); return a + b; }
 
 // ---------------------------------------------------------------- LDS access

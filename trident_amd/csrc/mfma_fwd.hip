@@ -118,6 +118,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
 
     f32x16 oacc[DB];
     float m, l;  // reference exponent (log2 domain, scaled) and this lane's partial sum
+    float m_use;  // m, or 0 while no key has been seen (m = -inf): what the exponents are taken against; follows m
     const float c = p.scale_log2;
 
     char* mask_lds = smem + kStages * kStageBytes + wave * kMaskBytes;
@@ -269,7 +270,8 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     float m_def = 0.f;   // the reference exponent they are taken against
     float c_def = c;     // the factor they are still to be multiplied by (1 where the mask has been added: scaled already)
     const uint32_t one2 = Mma<T>::pack2(1.f, 1.f);
-    const u32x4 ones = {one2, one2, one2, one2};
+    u32x4 ones = {one2, one2, one2, one2};
+    asm volatile("" : "+v"(ones));  // (kept in registers: as a constant it would be made anew from scalars in every tile)
     f32x16 lacc = zero16();
     auto frag = [&](auto with_pv, int j, int s) {
         constexpr int pv = decltype(with_pv)::value ? kPvSteps : 0;
@@ -331,6 +333,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     for (int db = 0; db < DB; ++db) oacc[db] = zero16();
     lacc = zero16();
     m = -INFINITY;
+    m_use = 0.f;
     l = 0.f;
     // tile 0 has landed and is visible to all waves (a later item's requests are older than the stores of the
     // item before it: everything is awaited)
@@ -394,13 +397,15 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
                     x[e] = key < p.S ? x[e] : -INFINITY;
                 }
             }
-            float mx = x[0], mx1 = x[16];  // two chains: a dependent maximum waits out the ALU latency
+            // two chains (a dependent maximum waits out the ALU latency) of three-operand maxima, written out: through
+            // fmaxf the compiler first canonicalises the operands of each chain (a maximum of a value with itself)
+            float mx = max3(x[0], x[1], x[2]), mx1 = max3(x[16], x[17], x[18]);
 #pragma unroll
-            for (int e = 1; e < 16; ++e) {
-                mx = fmaxf(mx, x[e]);
-                mx1 = fmaxf(mx1, x[16 + e]);
+            for (int e = 3; e < 15; e += 2) {
+                mx = max3(mx, x[e], x[e + 1]);
+                mx1 = max3(mx1, x[16 + e], x[17 + e]);
             }
-            mx = max_xor32(fmaxf(mx, mx1));
+            mx = max_xor32(max3(mx, x[15], max3(mx1, x[31], x[31])));
             mx *= cc;
             // Lazy rescaling: m is the reference exponent of l and of the O accumulators, not
             // necessarily the running maximum. It is only moved (and O rescaled) when some row of
@@ -408,7 +413,8 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
             // that factor, which fp32 sums and 16-bit P hold without loss.
             if (__builtin_amdgcn_ballot_w64(mx > m + kTau) != 0) {
                 const float m_new = fmaxf(m, mx);
-                const float alpha = fast_exp2(m - (m_new == -INFINITY ? 0.f : m_new));
+                m_use = m_new == -INFINITY ? 0.f : m_new;
+                const float alpha = fast_exp2(m - m_use);
                 l *= alpha;
                 m = m_new;
 #pragma unroll
@@ -420,7 +426,6 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
                     for (int i = 0; i < 16; ++i) lacc[i] *= alpha;
                 }
             }
-            const float m_use = m == -INFINITY ? 0.f : m;
             // exponentials in four groups of eight keys (one B operand each); the remaining loads of the
             // next tile and the first fragment reads of the matrix phase (tile j has been visible since
             // the previous barrier) are issued between the groups, so that none of them queues
