@@ -42,6 +42,10 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     constexpr int kBM = 32 * NW;
     constexpr int kKBytes = Tile::kBytes;
     constexpr int kStageBytes = 2 * Tile::kBytes;  // K tile, V tile
+    // The ring holds the K tiles first and the V tiles behind them (slot st: K at st * kKBytes, V at kVRing + st * kKBytes):
+    // every slot of an operand then lies within the 64 KiB an LDS instruction's immediate offset reaches from the lane's
+    // fragment address, and with the tile loop unrolled over the slots no fragment read needs address arithmetic.
+    constexpr int kVRing = kStages * Tile::kBytes;
     constexpr int kBlocksPerWave = 2 * Tile::kBlocks / NW;  // LDS-direct loads per wave and tile
     constexpr int KK = D / 16;  // K-steps of S^T
     constexpr int DB = D / 32;  // 32-row blocks of O^T
@@ -63,7 +67,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     // passes behind the epilogue. The epilogue's transposition patches then must not lie in ring stages 0-2.
     constexpr bool kPersistent = NW == 8 && MASK == kNoMask;
     using Store = RowBlockStore<T, 2>;                       // the epilogue stores 64 columns at a time
-    constexpr int kPatchOff = kPersistent ? 3 * kStageBytes : 0;
+    constexpr int kPatchOff = kPersistent ? kVRing + 3 * Tile::kBytes : 0;  // (behind the V tile of slot 2)
     constexpr int kRingBytes = kStages * kStageBytes;
     constexpr int kPatchEnd = kPatchOff + NW * Store::kPatchBytes;
     constexpr int kSmemBytes = (kPatchEnd > kRingBytes ? kPatchEnd : kRingBytes) + (kMaskViaLds ? NW * kMaskBytes : 0);
@@ -146,7 +150,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     const uint32_t voff = static_cast<uint32_t>(Tile::src_off(wave, lane, vrow_bytes));
     // load number idx (0 .. kBlocksPerWave-1) of this wave's share of tile t -> ring slot t % kStages
     auto issue_load = [&](int t, int idx) {
-        char* stage = smem + (t % kStages) * kStageBytes + wave * 1024;
+        char* stage = smem + (t % kStages) * kKBytes + wave * 1024;
         const int i = idx % kPerOperand;
         if (RAGGED && (t + 1) * kBN > p.S) {  // the sequence ends inside this tile: clamped rows, offsets from the tile's first row
             const int last = p.S - 1 - t * kBN;
@@ -155,11 +159,11 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
                                   Tile::src_off_clamped(wave + i * NW, lane, krow_bytes, last), stage + i * NW * 1024);
             else
                 lds_direct_load16(vbase + static_cast<int64_t>(t) * kBN * vrow_bytes,
-                                  Tile::src_off_clamped(wave + i * NW, lane, vrow_bytes, last), stage + kKBytes + i * NW * 1024);
+                                  Tile::src_off_clamped(wave + i * NW, lane, vrow_bytes, last), stage + kVRing + i * NW * 1024);
         } else if (idx < kPerOperand)
             lds_direct_load16(kbase + (static_cast<int64_t>(t) * kBN + i * kRowStep) * krow_bytes, koff, stage + i * NW * 1024);
         else
-            lds_direct_load16(vbase + (static_cast<int64_t>(t) * kBN + i * kRowStep) * vrow_bytes, voff, stage + kKBytes + i * NW * 1024);
+            lds_direct_load16(vbase + (static_cast<int64_t>(t) * kBN + i * kRowStep) * vrow_bytes, voff, stage + kVRing + i * NW * 1024);
     };
     // The loads of a tile are issued in four slices spread over the softmax phase: a wave stalls on a
     // load until the memory pipeline accepts it, and sixteen loads arriving at once from the four
@@ -198,7 +202,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     request_first_tiles();
 
     int row_off0 = Tile::off(l32, h);
-    int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
+    int tr_off0 = kVRing + Tile::tr_off(0, 0, lane), tr_off1 = kVRing + Tile::tr_off(0, 1, lane);  // (from the K ring's slot st)
     // fragment s of the S^T operand (key block s / KK, K-step s % KK) and of the O^T operand
     // (K-step s / DB = 16 keys, column block s % DB)
     auto k_frag = [&](const char* sK, int s) { return lds_read16(sK, (row_off0 ^ ((s % KK) << 5)) + 32 * (s / KK) * Tile::kRowBytes); };
@@ -273,13 +277,12 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     u32x4 ones = {one2, one2, one2, one2};
     asm volatile("" : "+v"(ones));  // (kept in registers: as a constant it would be made anew from scalars in every tile)
     f32x16 lacc = zero16();
-    auto frag = [&](auto with_pv, int j, int s) {
+    // (st: the ring slot of tile j, a literal at every call)
+    auto frag = [&](auto with_pv, int st, int s) __attribute__((always_inline)) {
         constexpr int pv = decltype(with_pv)::value ? kPvSteps : 0;
-        const char* stage_j = smem + ((j + kStages) % kStages) * kStageBytes;
-        const char* stage_n = smem + ((j + 1) % kStages) * kStageBytes;
-        return s < pv ? v_frag(stage_j + kKBytes, s) : k_frag(stage_n, s - pv);
+        return s < pv ? v_frag(smem + st * kKBytes, s) : k_frag(smem + ((st + 1) % kStages) * kKBytes, s - pv);
     };
-    auto matrix_phase = [&](auto with_pv, auto with_s, int j, bool do_s = true) {
+    auto matrix_phase = [&](auto with_pv, auto with_s, int st, bool do_s = true) __attribute__((always_inline)) {
         constexpr int pv = decltype(with_pv)::value ? kPvSteps : 0;
         constexpr int total = pv + (decltype(with_s)::value ? kSteps : 0);
         if constexpr (decltype(with_s)::value) {
@@ -299,7 +302,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
             }
             if (s + kRing < total) {
                 const int n = s + kRing;
-                ring[s % kRing] = frag(with_pv, j, n);
+                ring[s % kRing] = frag(with_pv, st, n);
             }
             if constexpr (kDefer && pv > 0) {
                 // group 2 (B operand of K-step 2, first used at step 2 DB) during steps 0 .. 2 DB - 1,
@@ -351,15 +354,16 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     {
         load_mask(0);
 #pragma unroll
-        for (int r = 0; r < kRing; ++r) ring[r] = frag(No{}, -1, r);
+        for (int r = 0; r < kRing; ++r) ring[r] = frag(No{}, kStages - 1, r);
         __builtin_amdgcn_sched_barrier(0);
-        matrix_phase(No{}, Yes{}, -1);
+        matrix_phase(No{}, Yes{}, kStages - 1);
         take_mask_block(0, true, false);
     }
 
     // A wave computes on its first my_tiles tiles (all of them without a causal mask) and afterwards
     // only keeps fetching its share of the remaining tiles and meeting the barriers.
-    for (int j = 0; j < my_tiles; ++j) {
+    // One step of the tile loop; st = j % kStages is a literal at each of the loop's four calls.
+    auto tile_step = [&](const int j, const int st) __attribute__((always_inline)) {
         // slot of tile j+dist: every wave is done with the tile it held (two barriers ago at the latest)
         const bool issued = j + dist < n_tiles;
         if (issued) issue_slice(j + dist, 0);
@@ -442,7 +446,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
                 if (ks < 2 && issued) issue_slice(j + dist, 2 + ks);
                 if (ks < 2) {
 #pragma unroll
-                    for (int r = kRing / 2 * ks; r < kRing / 2 * (ks + 1); ++r) ring[r] = frag(Yes{}, j, r);
+                    for (int r = kRing / 2 * ks; r < kRing / 2 * (ks + 1); ++r) ring[r] = frag(Yes{}, st, r);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -502,7 +506,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
             // the few instructions of this phase go first, so that the matrix pipe never waits for an
             // issue slot behind the partner's vector work
             __builtin_amdgcn_s_setprio(2);
-            matrix_phase(Yes{}, Yes{}, j, with_s || DROPOUT);
+            matrix_phase(Yes{}, Yes{}, st, with_s || DROPOUT);
             __builtin_amdgcn_s_setprio(0);
             if (with_s) take_mask_block(j + 1, false, issued);
         }
@@ -511,6 +515,20 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
             lds_barrier();
             __builtin_amdgcn_sched_barrier(0);
         }
+    };
+    static_assert(kStages == 4, "the tile loop is unrolled over the ring's slots");
+    // (a mask and dropout together at D = 128 have no registers to spare for four copies of the step: rolled, the slot
+    // is a run-time value there and every fragment read adds it to its address)
+    constexpr bool kUnrolled = !(D == 128 && MASK != kNoMask && DROPOUT);
+    if constexpr (kUnrolled) {
+        for (int j = 0; j < my_tiles; j += 4) {
+            tile_step(j, 0);
+            if (j + 1 < my_tiles) tile_step(j + 1, 1);
+            if (j + 2 < my_tiles) tile_step(j + 2, 2);
+            if (j + 3 < my_tiles) tile_step(j + 3, 3);
+        }
+    } else {
+        for (int j = 0; j < my_tiles; ++j) tile_step(j, j % kStages);
     }
     for (int j = my_tiles; j < n_tiles; ++j) {
         const bool issued = j + dist < n_tiles;
