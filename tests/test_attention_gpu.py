@@ -188,7 +188,7 @@ def test_key_padding_mask_row_broadcast(dtype, D, S, p, device):
                                                      (torch.float16, torch.float16, (1, 3, 256, 256)),
                                                      (torch.bfloat16, torch.float32, (2, 1, 1, 256)),
                                                      (torch.float32, torch.float32, (1, 1, 1, 256))])
-@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("D", [32, 64, 128])
 def test_mask_gradient_on_the_matrix_cores(dtype, mask_dtype, mshape, D, device):
     """The mask gradient from the matrix-core dQ kernel (16-bit problems): written in place for a full mask, added
     atomically into the mask's own shape for masks broadcast over batch, heads or rows (a key-padding mask with a
@@ -209,7 +209,7 @@ def test_mask_gradient_on_the_matrix_cores(dtype, mask_dtype, mshape, D, device)
     assert _lib.lib().tri_attn_uses_matrix_cores(ctypes.byref(args), 2) == (2 if dtype == torch.float32 else 1)
 
 
-@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("D", [32, 64, 128])
 def test_fp32_mask_many_tiles(D, device):
     """fp32 mask shared by the heads over 8 key tiles and 2 workgroups per head: the staged mask path (D=64)
     refills its LDS region every tile; D=128 takes the direct loads."""
@@ -278,7 +278,8 @@ def test_dropout_mask_bits_match_oracle(device):
 
 
 @pytest.mark.parametrize("dtype,S,D", [(torch.float32, 64, 32), (torch.bfloat16, 256, 128), (torch.float16, 128, 64),
-                                       (torch.bfloat16, 512, 64), (torch.float16, 512, 128)])
+                                       (torch.bfloat16, 512, 64), (torch.float16, 512, 128), (torch.bfloat16, 512, 32),
+                                       (torch.float16, 128, 32)])
 @pytest.mark.parametrize("p", [0.1, 0.5])
 def test_dropout_forward_backward(dtype, S, D, p, device):
     q, k, v, d_o = _gen((2, 2, S, D), 61, dtype)
@@ -361,7 +362,7 @@ def _abi_case(device, dtype, S, D, variant, seed, batches=1, heads=2, matrix_cor
 
 
 @pytest.mark.parametrize("variant", ["plain", "causal", "mask", "mask16", "causal+dropout"])
-@pytest.mark.parametrize("S,D", [(384, 64), (384, 128), (640, 64), (640, 128)])
+@pytest.mark.parametrize("S,D", [(384, 64), (384, 128), (640, 64), (640, 128), (384, 32), (640, 32)])
 def test_four_wave_kernels_over_several_tiles(S, D, variant, device):
     _abi_case(device, torch.bfloat16, S, D, variant, 200 + S + D)
 
@@ -373,10 +374,10 @@ def test_lengths_that_are_not_powers_of_two(dtype, S, D, variant, device):
     _abi_case(device, dtype, S, D, variant, 300 + S + D)
 
 
-@pytest.mark.parametrize("S,D", [(256, 64), (256, 128), (512, 64), (512, 128), (384, 128)])
+@pytest.mark.parametrize("S,D", [(256, 64), (256, 128), (512, 64), (512, 128), (384, 128), (512, 32), (384, 32)])
 def test_dropout_without_causal_or_mask(S, D, device):
     """Dropout alone: the persistent forward kernel, the D = 128 unphased dQ kernel, the phased dQ kernel at
-    D = 64 and the D = 128 pair dK/dV kernel in their non-causal dropout instantiations."""
+    D = 64 and 32 and the D = 128 pair dK/dV kernel in their non-causal dropout instantiations."""
     _abi_case(device, torch.bfloat16, S, D, "dropout", 250 + S + D)
 
 
@@ -407,7 +408,8 @@ def test_operator_without_the_reference_limits(dtype, S, D, device):
 @pytest.mark.parametrize("dtype,S,D", [(torch.float16, 32, 64), (torch.bfloat16, 64, 64), (torch.bfloat16, 32, 128),
                                        (torch.float16, 72, 64), (torch.bfloat16, 200, 128), (torch.bfloat16, 129, 64),
                                        (torch.float16, 255, 128), (torch.bfloat16, 1000, 64), (torch.bfloat16, 1, 64),
-                                       (torch.float16, 833, 128)])
+                                       (torch.float16, 833, 128), (torch.bfloat16, 32, 32), (torch.float16, 333, 32),
+                                       (torch.bfloat16, 1, 32)])
 def test_any_length_runs_on_the_matrix_cores(dtype, S, D, variant, device):
     """Lengths that are not multiples of 128 (the reference's benchmark regime S = 32, 64 among them): the 128-row
     matrix-core kernels with boundary handling (clamped loads, masked keys and rows, guarded stores), not the
@@ -416,11 +418,12 @@ def test_any_length_runs_on_the_matrix_cores(dtype, S, D, variant, device):
 
 
 def test_what_the_16_bit_kernels_leave_runs_on_the_32_row_tile_kernels(device):
-    """Masked problems of other lengths, fp32 problems and small heads: family 2 (v_mfma_f32_32x32x2_f32 for fp32 data,
-    the 16-bit 32x32x8 instruction for 16-bit data) in all three passes."""
+    """Masked problems of other lengths, fp32 problems and the smallest head: family 2 (v_mfma_f32_32x32x2_f32 for fp32
+    data, the 16-bit 32x32x8 instruction for 16-bit data) in all three passes; a 16-bit head of 32 is family 1."""
     _abi_case(device, torch.bfloat16, 200, 64, "mask", 650, matrix_cores=[2, 2, 2])
     _abi_case(device, torch.float32, 256, 64, "plain", 651, matrix_cores=[2, 2, 2])
-    _abi_case(device, torch.bfloat16, 256, 32, "causal", 652, matrix_cores=[2, 2, 2])
+    _abi_case(device, torch.bfloat16, 256, 16, "causal", 652, matrix_cores=[2, 2, 2])
+    _abi_case(device, torch.bfloat16, 256, 32, "causal", 653, matrix_cores=[1, 1, 1])
 
 
 @pytest.mark.parametrize("variant", ["plain", "causal", "mask", "mask16", "dropout", "causal+dropout"])
@@ -434,7 +437,9 @@ def test_32_row_tile_kernels(dtype, S, D, variant, device):
     size, over lengths with a ragged last tile (and one of a single row), three heads, every mask mode and dropout."""
     if variant == "mask16" and dtype == torch.float32:
         pytest.skip("a 16-bit mask is a mask of the operand type")
-    _abi_case(device, dtype, S, D, variant, 700 + S + D, batches=2 if S < 300 else 1, heads=3, matrix_cores=[2, 2, 2])
+    # (a 16-bit head of 32 without a mask is the 64-key-tile kernels' at any length)
+    family = 1 if dtype != torch.float32 and D == 32 and "mask" not in variant else 2
+    _abi_case(device, dtype, S, D, variant, 700 + S + D, batches=2 if S < 300 else 1, heads=3, matrix_cores=[family] * 3)
 
 
 def test_32_row_tile_kernels_masked_16_bit_lengths(device):
@@ -500,7 +505,7 @@ def test_random_problems(dtype, S, D, variant, batches, heads, seed, device):
 
 # ------------------------------------------------------------------ tile counts of the phased kernels
 @pytest.mark.parametrize("variant", ["plain", "causal", "causal+dropout"])
-@pytest.mark.parametrize("S,D", [(256, 128), (768, 128), (1280, 128), (768, 64), (1024, 64)])
+@pytest.mark.parametrize("S,D", [(256, 128), (768, 128), (1280, 128), (768, 64), (1024, 64), (256, 32), (1280, 32)])
 def test_phased_kernels_over_tile_counts(S, D, variant, device):
     """Multiples of 256 that are not powers of two included (the operator API cannot pass those): 4 to 20
     streamed tiles, so the prologue, the steady state and the drain of the load pipeline of the forward
@@ -509,7 +514,7 @@ def test_phased_kernels_over_tile_counts(S, D, variant, device):
 
 
 @pytest.mark.parametrize("variant", ["plain", "causal", "causal+dropout"])
-@pytest.mark.parametrize("batches,heads,S,D", [(4, 40, 512, 128), (3, 31, 768, 64), (8, 8, 1280, 128)])
+@pytest.mark.parametrize("batches,heads,S,D", [(4, 40, 512, 128), (3, 31, 768, 64), (8, 8, 1280, 128), (5, 31, 768, 32)])
 def test_more_items_than_compute_units(batches, heads, S, D, variant, device):
     """More (head, row tile) items than the GPU has compute units (320, 279 and 320 against 256): the
     persistent forward workgroups each walk two items, with the items dealt per XCD when the head count is a
@@ -519,7 +524,8 @@ def test_more_items_than_compute_units(batches, heads, S, D, variant, device):
 
 # ------------------------------------------------------------------ the combined backward entry point
 @pytest.mark.parametrize("S,D,causal,p", [(512, 128, True, 0.0), (256, 64, False, 0.0), (512, 64, True, 0.25),
-                                          (256, 128, True, 0.25), (384, 128, True, 0.0)])
+                                          (256, 128, True, 0.25), (384, 128, True, 0.0), (512, 32, True, 0.0),
+                                          (384, 32, False, 0.25)])
 def test_combined_backward_matches_the_three_calls(S, D, causal, p, device):
     """tri_attn_bwd may fold the delta pre-pass into the dQ kernel and reorder the launches; its
     results must be those of delta, dK/dV and dQ called one after the other."""
@@ -649,7 +655,7 @@ def test_mask_block_classes(mshape, mask_dtype, device):
     assert torch.equal(got[:size].reshape(kinds.shape).long(), kinds)
 
 
-@pytest.mark.parametrize("D,p", [(64, 0.0), (128, 0.0), (64, 0.3)])
+@pytest.mark.parametrize("D,p", [(64, 0.0), (128, 0.0), (64, 0.3), (32, 0.0)])
 def test_classes_do_not_change_results(D, p, device):
     """The same calls with and without mask_classes give the same results: skipped tiles only ever added zeros."""
     import ctypes
@@ -694,7 +700,7 @@ def test_classes_do_not_change_results(D, p, device):
                 assert (a32 != b32).float().mean().item() < 0.2, (kind, name)
 
 
-@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("D", [32, 64, 128])
 def test_dense_mask_gradient_behind_the_last_active_tile(D, device):
     """A full-shape mask whose trailing key blocks are all -inf, with a gradient: the block classes let the kernels
     stop streaming behind the last active tile, but the mask gradient written in place must still cover every tile
@@ -744,7 +750,7 @@ def test_dense_mask_gradient_behind_the_last_active_tile(D, device):
     _check(device, dtype, q, k, v, d_o, mask=mask, mask_grad=True, tag="operator dmask")
 
 
-@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("D", [32, 64, 128])
 def test_mask_written_between_two_calls(D, device):
     """The operator keeps the block classes of a mask tensor between calls; writing to the tensor (version counter)
     must bring fresh ones: the second mask opens keys the first one had masked out."""

@@ -1,4 +1,4 @@
-// Backward attention on the matrix cores for fp16/bf16, D in {64,128}, S a multiple of 128
+// Backward attention on the matrix cores for fp16/bf16, D in {32,64,128}, S a multiple of 128
 // (replaces trident/kernel/attention.py:169-339, split in two passes so that no gradient
 // tile is ever accumulated in global memory):
 //
@@ -56,7 +56,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
     // A mask block of a wave (32 rows x 64 keys) goes through a private LDS region (8 KiB fp32, 4 KiB for a mask of
     // the operand type) when it fits (D = 64): lanes own rows, so direct loads would touch 32 cache lines per
     // instruction, while LDS-direct loads fetch whole rows. Geometry of a 32-row SwzTile<128> / SwzTile<64>.
-    constexpr bool kMaskViaLds = MASK != kNoMask && D == 64;  // (at D = 128 the 4 KiB regions of a 16-bit mask would fit, but the kernel then spills)
+    constexpr bool kMaskViaLds = MASK != kNoMask && D <= 64;  // (at D = 128 the 4 KiB regions of a 16-bit mask would fit, but the kernel then spills)
     constexpr int kMaskElt = MASK == kMaskF32 ? 4 : 2;
     using MaskTile = std::conditional_t<MASK == kMaskF32, SwzTile<128>, SwzTile<64>>;
     constexpr int kMaskBytes = 32 * MaskTile::kRowBytes;
@@ -335,12 +335,15 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
     constexpr int KK = D / 16;
     constexpr int DB = D / 32;
     constexpr int kBlocksPerWave = 2 * Tile::kBlocks / NW;
-    constexpr int kPerOperand = Tile::kBlocks / NW;
+    // (D = 32: a tile has four blocks per operand, waves 0-3 fetch the K tile's and waves 4-7 the V tile's)
+    constexpr bool kSplitOperands = Tile::kBlocks < NW;
+    constexpr int kPerOperand = kSplitOperands ? 1 : Tile::kBlocks / NW;
     constexpr int kRowStep = NW * Tile::kRowsPerBlock;
-    static_assert(kRowStep % 16 == 0 && 2 * kPerOperand == kBlocksPerWave, "block assignment");
+    static_assert(kRowStep % 16 == 0 && (kSplitOperands ? kBlocksPerWave == 1 && 2 * Tile::kBlocks == NW : 2 * kPerOperand == kBlocksPerWave),
+                  "block assignment");
     constexpr int kDqSteps = 4 * DB;           // MFMAs of dQ^T per tile
     constexpr int kSteps = kDqSteps + 4 * KK;  // + S^T and dP^T of the next tile
-    constexpr int kRing = DROPOUT && D == 128 ? 4 : 6;  // (registers)
+    constexpr int kRing = (DROPOUT && D == 128) || D == 32 ? 4 : 6;  // (registers; at D = 32 the dQ^T steps are four)
     static_assert(kRing <= kDqSteps, "the vector phase requests dQ fragments only");
     // The workgroup's Q and dO rows reach the registers through LDS as well: lanes own rows, so direct loads
     // touch 32 cache lines per instruction, while LDS-direct loads fetch whole rows. Each wave stages its
@@ -392,10 +395,16 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
 
     // A wave fetches blocks wave, wave + NW, ... of the K tile and of the V tile: their rows are a
     // multiple of 16 apart, so one per-lane source offset serves all of them.
-    const uint32_t koff = static_cast<uint32_t>(Tile::src_off(wave, lane, krow_bytes));
-    const uint32_t voff = static_cast<uint32_t>(Tile::src_off(wave, lane, vrow_bytes));
+    const int my_block = kSplitOperands ? wave % Tile::kBlocks : wave;
+    const uint32_t koff = static_cast<uint32_t>(Tile::src_off(my_block, lane, krow_bytes));
+    const uint32_t voff = static_cast<uint32_t>(Tile::src_off(my_block, lane, vrow_bytes));
     auto issue_tile = [&](int t) {
-        char* stage = smem + (t % kStages) * kStageBytes + wave * 1024;
+        char* stage = smem + (t % kStages) * kStageBytes + my_block * 1024;
+        if constexpr (kSplitOperands) {
+            if (wave < Tile::kBlocks) lds_direct_load16(kbase + static_cast<int64_t>(t) * kBN * krow_bytes, koff, stage);
+            else lds_direct_load16(vbase + static_cast<int64_t>(t) * kBN * vrow_bytes, voff, stage + Tile::kBytes);
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < kPerOperand; ++i)
             lds_direct_load16(kbase + (static_cast<int64_t>(t) * kBN + i * kRowStep) * krow_bytes, koff, stage + i * NW * 1024);
@@ -610,7 +619,7 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
     // of the operand type) when it fits (D = 64). Plain loads would be tracked by the compiler, whose waits for them
     // also drain the LDS-direct tile loads issued in between (the counter completes in order), which makes the
     // tile prefetch synchronous. Geometry of a 64-row SwzTile<64> / SwzTile<32> (128- or 64-byte rows = 32 keys).
-    constexpr bool kMaskViaLds = MASK != kNoMask && D == 64;
+    constexpr bool kMaskViaLds = MASK != kNoMask && D <= 64;
     constexpr int kMaskElt = MASK == kMaskF32 ? 4 : 2;
     using MaskTile = std::conditional_t<MASK == kMaskF32, SwzTile<64>, SwzTile<32>>;
     constexpr int kMaskLoads = MaskTile::kBlocks;
@@ -1715,7 +1724,7 @@ int launch_dq_waves(const KParams& p, hipStream_t stream) {
 // its registers only under the causal mask and with a fragment ring of 4)
 template <int D, int MASK>
 bool dq_is_phased(const KParams& p) {
-    return MASK == kNoMask && p.S % 256 == 0 && (D == 64 || p.thr8 <= 0 || p.causal);
+    return MASK == kNoMask && p.S % 256 == 0 && (D <= 64 || p.thr8 <= 0 || p.causal);
 }
 
 template <typename T, int D, bool CAUSAL, int MASK>
@@ -1723,7 +1732,7 @@ int launch_dq_dropout(const KParams& p, hipStream_t stream, bool with_delta) {
     if constexpr (MASK == kNoMask) {
         if (dq_is_phased<D, MASK>(p)) {
             const dim3 grid(p.B * p.H * (p.S / 256)), block(512);
-            if constexpr (D == 64 || CAUSAL) {
+            if constexpr (D <= 64 || CAUSAL) {
                 if (p.thr8 > 0) {
                     if (with_delta) hipLaunchKernelGGL((mfma_dq_phased_kernel<T, D, CAUSAL, true, true>), grid, block, 0, stream, p);
                     else hipLaunchKernelGGL((mfma_dq_phased_kernel<T, D, CAUSAL, true, false>), grid, block, 0, stream, p);
@@ -1769,7 +1778,7 @@ int launch_dkdv_dropout(const KParams& p, hipStream_t stream) {
         }
         return TRI_ATTN_ESHAPE;  // (mfma_supported keeps masked problems of such lengths away)
     }
-    if constexpr (D == 64) {
+    if constexpr (D <= 64) {
         // the two-waves-per-SIMD kernel fits its registers: 8 waves (256 keys) when the sequence
         // allows it, else 4 waves (128 keys)
         if (p.S % 256 == 0) return launch_dkdv_waves<T, D, 8, CAUSAL, MASK>(p, stream);
@@ -1815,13 +1824,17 @@ int launch_bwd_variant(int dtype, const KParams& p, hipStream_t stream, bool wit
     return TRI_ATTN_EDTYPE;
 }
 
+template <int WHICH, typename T>
+int launch_bwd_head(int dtype, const KParams& p, hipStream_t stream, bool with_delta) {
+    if (p.D == 128) return launch_bwd_variant<WHICH, T, 128>(dtype, p, stream, with_delta);
+    if (p.D == 64) return launch_bwd_variant<WHICH, T, 64>(dtype, p, stream, with_delta);
+    return launch_bwd_variant<WHICH, T, 32>(dtype, p, stream, with_delta);
+}
+
 template <int WHICH>
 int launch_bwd(int dtype, const KParams& p, hipStream_t stream, bool with_delta) {
-    if (dtype == TRI_ATTN_BF16)
-        return p.D == 128 ? launch_bwd_variant<WHICH, bf16_t, 128>(dtype, p, stream, with_delta)
-                          : launch_bwd_variant<WHICH, bf16_t, 64>(dtype, p, stream, with_delta);
-    return p.D == 128 ? launch_bwd_variant<WHICH, f16_t, 128>(dtype, p, stream, with_delta)
-                      : launch_bwd_variant<WHICH, f16_t, 64>(dtype, p, stream, with_delta);
+    return dtype == TRI_ATTN_BF16 ? launch_bwd_head<WHICH, bf16_t>(dtype, p, stream, with_delta)
+                                  : launch_bwd_head<WHICH, f16_t>(dtype, p, stream, with_delta);
 }
 
 }  // namespace

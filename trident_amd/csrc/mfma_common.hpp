@@ -175,7 +175,7 @@ struct SwzTile {
     // land in distinct banks
     static __device__ __forceinline__ int swz(int r) {
         if constexpr (D == 128) return ((r & 7) << 1) | ((r >> 3) & 1);
-        else if constexpr (D == 32) return (r >> 1) & 3;  // (64-byte rows, four chunks: mask blocks of 16-bit values)
+        else if constexpr (D == 32) return (r >> 2) & 3;  // (64-byte rows, four chunks: four rows fill the 64 banks once)
         else return (((r >> 1) & 3) << 1) | ((r >> 3) & 1);
     }
     static __device__ __forceinline__ int off(int r, int c) { return r * kRowBytes + ((c ^ swz(r)) << 4); }

@@ -1,5 +1,5 @@
 // Forward attention on the matrix cores: online-softmax flash kernel for fp16/bf16,
-// D in {64,128}; any S without a mask, multiples of 128 with one (replaces trident/kernel/attention.py:33-165).
+// D in {32,64,128}; any S without a mask, multiples of 128 with one (replaces trident/kernel/attention.py:33-165).
 //
 // A workgroup of NW waves owns 32*NW query rows, one wave 32 of them. Q stays in registers as
 // the B operand of S^T = K Q^T; K and V tiles of 64 keys live row-major (swizzled) in a four-stage
@@ -47,6 +47,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     // fragment address, and with the tile loop unrolled over the slots no fragment read needs address arithmetic.
     constexpr int kVRing = kStages * Tile::kBytes;
     constexpr int kBlocksPerWave = 2 * Tile::kBlocks / NW;  // LDS-direct loads per wave and tile
+    static_assert(kBlocksPerWave >= 1, "every wave fetches a piece of every tile");
     constexpr int KK = D / 16;  // K-steps of S^T
     constexpr int DB = D / 32;  // 32-row blocks of O^T
     constexpr int kSteps = 2 * KK;    // MFMAs of S^T per tile
@@ -57,7 +58,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     // for one of the operand type) when it fits (D = 64): lanes own rows, so direct loads would touch 32 cache
     // lines per instruction, while LDS-direct loads fetch whole rows (256 or 128 bytes) and the swizzled tile is
     // read back 16 or 8 bytes at a time. The region has the geometry of a 32-row SwzTile<128> / SwzTile<64>.
-    constexpr bool kMaskViaLds = MASK != kNoMask && (D == 64 || (MASK == kMaskT && NW == 8 && !DROPOUT));  // (D = 128: 4 KiB regions fit, 8 KiB ones do not; with dropout the registers for the staged values are not there)
+    constexpr bool kMaskViaLds = MASK != kNoMask && (D <= 64 || (MASK == kMaskT && NW == 8 && !DROPOUT));  // (D = 128: 4 KiB regions fit, 8 KiB ones do not; with dropout the registers for the staged values are not there)
     constexpr int kMaskElt = MASK == kMaskF32 ? 4 : 2;
     using MaskTile = std::conditional_t<MASK == kMaskF32, SwzTile<128>, SwzTile<64>>;
     constexpr int kMaskBytes = 32 * MaskTile::kRowBytes;
@@ -66,7 +67,8 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     // one, so that a new item's memory latency (6 000-9 000 cycles from a workgroup's entry to its first rows)
     // passes behind the epilogue. The epilogue's transposition patches then must not lie in ring stages 0-2.
     constexpr bool kPersistent = NW == 8 && MASK == kNoMask;
-    using Store = RowBlockStore<T, 2>;                       // the epilogue stores 64 columns at a time
+    constexpr int kStoreBlocks = DB >= 2 ? 2 : 1;
+    using Store = RowBlockStore<T, kStoreBlocks>;            // the epilogue stores 64 columns at a time (32 at D = 32)
     constexpr int kPatchOff = kPersistent ? kVRing + 3 * Tile::kBytes : 0;  // (behind the V tile of slot 2)
     constexpr int kRingBytes = kStages * kStageBytes;
     constexpr int kPatchEnd = kPatchOff + NW * Store::kPatchBytes;
@@ -143,14 +145,23 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     // A wave fetches blocks wave, wave + NW, ... of the K tile and of the V tile: their rows are a
     // multiple of 16 apart, so one per-lane source offset (row within the block, swizzled chunk)
     // serves all of them and the rest of the address is scalar arithmetic.
-    constexpr int kPerOperand = Tile::kBlocks / NW;
+    // (D = 32 with 8 waves: a tile has four blocks per operand, waves 0-3 fetch the K tile's and waves 4-7 the V tile's)
+    constexpr bool kSplitOperands = Tile::kBlocks < NW;
+    constexpr int kPerOperand = kSplitOperands ? 1 : Tile::kBlocks / NW;
     constexpr int kRowStep = NW * Tile::kRowsPerBlock;
-    static_assert(kRowStep % 16 == 0 && 2 * kPerOperand == kBlocksPerWave, "block assignment");
-    const uint32_t koff = static_cast<uint32_t>(Tile::src_off(wave, lane, krow_bytes));
-    const uint32_t voff = static_cast<uint32_t>(Tile::src_off(wave, lane, vrow_bytes));
+    static_assert(kRowStep % 16 == 0 && (kSplitOperands ? kBlocksPerWave == 1 && 2 * Tile::kBlocks == NW : 2 * kPerOperand == kBlocksPerWave),
+                  "block assignment");
+    const int my_block = kSplitOperands ? wave % Tile::kBlocks : wave;
+    const uint32_t koff = static_cast<uint32_t>(Tile::src_off(my_block, lane, krow_bytes));
+    const uint32_t voff = static_cast<uint32_t>(Tile::src_off(my_block, lane, vrow_bytes));
     // load number idx (0 .. kBlocksPerWave-1) of this wave's share of tile t -> ring slot t % kStages
     auto issue_load = [&](int t, int idx) {
-        char* stage = smem + (t % kStages) * kKBytes + wave * 1024;
+        char* stage = smem + (t % kStages) * kKBytes + my_block * 1024;
+        if constexpr (kSplitOperands) {
+            if (wave < Tile::kBlocks) lds_direct_load16(kbase + static_cast<int64_t>(t) * kBN * krow_bytes, koff, stage);
+            else lds_direct_load16(vbase + static_cast<int64_t>(t) * kBN * vrow_bytes, voff, stage + kVRing);
+            return;
+        }
         const int i = idx % kPerOperand;
         if (RAGGED && (t + 1) * kBN > p.S) {  // the sequence ends inside this tile: clamped rows, offsets from the tile's first row
             const int last = p.S - 1 - t * kBN;
@@ -354,7 +365,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     {
         load_mask(0);
 #pragma unroll
-        for (int r = 0; r < kRing; ++r) ring[r] = frag(No{}, kStages - 1, r);
+        for (int r = 0; r < (kRing < kSteps ? kRing : kSteps); ++r) ring[r] = frag(No{}, kStages - 1, r);
         __builtin_amdgcn_sched_barrier(0);
         matrix_phase(No{}, Yes{}, kStages - 1);
         take_mask_block(0, true, false);
@@ -555,12 +566,12 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
         }
     }
     {
-        static_assert(DB % 2 == 0, "64 columns per store");
+        static_assert(DB % kStoreBlocks == 0, "whole stores");
         char* patch = smem + kPatchOff + wave * Store::kPatchBytes;
 #pragma unroll
-        for (int cb = 0; cb < DB / 2; ++cb) {
+        for (int cb = 0; cb < DB / kStoreBlocks; ++cb) {
             if (cb) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // patch read before it is rewritten
-            const f32x16(&part)[2] = *reinterpret_cast<const f32x16(*)[2]>(&oacc[2 * cb]);
+            const f32x16(&part)[kStoreBlocks] = *reinterpret_cast<const f32x16(*)[kStoreBlocks]>(&oacc[kStoreBlocks * cb]);
             Store::run(part, [inv](float x) { return x * inv; }, patch, o0 + cb * 128, p.os[2] * 2, lane,
                        RAGGED ? p.S - wrow0 : 32);
         }
@@ -608,10 +619,15 @@ int launch_fwd_waves(int dtype, const KParams& p, hipStream_t stream) {
 
 }  // namespace
 
+template <typename T>
+int launch_fwd_head(int dtype, const KParams& p, hipStream_t stream) {
+    if (p.D == 128) return launch_fwd_waves<T, 128>(dtype, p, stream);
+    if (p.D == 64) return launch_fwd_waves<T, 64>(dtype, p, stream);
+    return launch_fwd_waves<T, 32>(dtype, p, stream);
+}
+
 int launch_mfma_fwd(int dtype, const KParams& p, hipStream_t stream) {
-    if (dtype == TRI_ATTN_BF16)
-        return p.D == 128 ? launch_fwd_waves<bf16_t, 128>(dtype, p, stream) : launch_fwd_waves<bf16_t, 64>(dtype, p, stream);
-    return p.D == 128 ? launch_fwd_waves<f16_t, 128>(dtype, p, stream) : launch_fwd_waves<f16_t, 64>(dtype, p, stream);
+    return dtype == TRI_ATTN_BF16 ? launch_fwd_head<bf16_t>(dtype, p, stream) : launch_fwd_head<f16_t>(dtype, p, stream);
 }
 
 }  // namespace tri
