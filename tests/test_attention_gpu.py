@@ -377,7 +377,7 @@ def test_lengths_that_are_not_powers_of_two(dtype, S, D, variant, device):
 @pytest.mark.parametrize("S,D", [(256, 64), (256, 128), (512, 64), (512, 128), (384, 128), (512, 32), (384, 32)])
 def test_dropout_without_causal_or_mask(S, D, device):
     """Dropout alone: the persistent forward kernel, the D = 128 unphased dQ kernel, the phased dQ kernel at
-    D = 64 and 32 and the D = 128 pair dK/dV kernel in their non-causal dropout instantiations."""
+    D = 64, the unphased one at D = 32 and the D = 128 pair dK/dV kernel in their non-causal dropout instantiations."""
     _abi_case(device, torch.bfloat16, S, D, "dropout", 250 + S + D)
 
 
@@ -520,6 +520,38 @@ def test_more_items_than_compute_units(batches, heads, S, D, variant, device):
     persistent forward workgroups each walk two items, with the items dealt per XCD when the head count is a
     multiple of 8 (a partly filled, reversed second round) and in launch order otherwise."""
     _abi_case(device, torch.bfloat16 if D == 128 else torch.float16, S, D, variant, 700 + S + D, batches, heads)
+
+
+@pytest.mark.parametrize("B,H,S,D,causal", [(8, 16, 896, 32, False), (8, 16, 2176, 32, True), (8, 16, 1024, 32, True),
+                                            (6, 16, 1152, 64, True)])
+def test_a_head_does_not_depend_on_its_company(B, H, S, D, causal, device):
+    """Several workgroups resident per compute unit (small heads: four 4-wave workgroups): every head of a launch with a
+    thousand workgroups gets bit for bit what it gets in a launch of its batch alone, and two heads match the oracle.
+    (A fragment of a tile requested before the barrier that publishes the tile shows up here, and only here: in small
+    launches the tile has always landed.)"""
+    from trident_amd.operation import Attention
+    dtype = torch.bfloat16
+    q, k, v, d_o = _gen((B, H, S, D), 4100 + S + D, dtype)
+    scale = 1.0 / math.sqrt(D)
+    tq, tk, tv, tdo = [x.to(device) for x in (q, k, v, d_o)]
+    o, lse = Attention._forward(tq, tk, tv, None, 0.0, causal, scale, 0, 0)
+    dq, dk, dv, _ = Attention._backward(tdo, tq, tk, tv, o, lse, None, scale, 0.0, causal, 0, 0, False)
+    for b in range(B):
+        sl = slice(b, b + 1)
+        o1, lse1 = Attention._forward(tq[sl], tk[sl], tv[sl], None, 0.0, causal, scale, 0, 0)
+        dq1, dk1, dv1, _ = Attention._backward(tdo[sl], tq[sl], tk[sl], tv[sl], o1, lse1, None, scale, 0.0, causal, 0, 0, False)
+        for name, whole, part in (("O", o, o1), ("LSE", lse, lse1), ("dQ", dq, dq1), ("dK", dk, dk1), ("dV", dv, dv1)):
+            assert torch.equal(whole[sl], part), f"{name} of batch {b} differs between the launches"
+    hs = slice(H - 2, H)
+    kw = dict(is_causal=causal, scale=scale)
+    qs, ks, vs, gs = [x[B - 1:, hs] for x in (q, k, v, d_o)]
+    o_ref, _ = parity.oracle_forward(qs, ks, vs, **kw)
+    parity.close(o[B - 1:, hs], o_ref, dtype, "company O")
+    dq_r, dk_r, dv_r, _, _ = parity.oracle_backward(qs, ks, vs, gs, o=o[B - 1:, hs], **kw)
+    _, a_dq, a_dk, a_dv = parity.oracle_abs_sums(qs, ks, vs, gs, o=o[B - 1:, hs], **kw)
+    parity.close(dq[B - 1:, hs], dq_r, dtype, "company dQ", a_dq)
+    parity.close(dk[B - 1:, hs], dk_r, dtype, "company dK", a_dk)
+    parity.close(dv[B - 1:, hs], dv_r, dtype, "company dV", a_dv)
 
 
 # ------------------------------------------------------------------ the combined backward entry point

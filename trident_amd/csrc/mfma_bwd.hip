@@ -335,15 +335,12 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
     constexpr int KK = D / 16;
     constexpr int DB = D / 32;
     constexpr int kBlocksPerWave = 2 * Tile::kBlocks / NW;
-    // (D = 32: a tile has four blocks per operand, waves 0-3 fetch the K tile's and waves 4-7 the V tile's)
-    constexpr bool kSplitOperands = Tile::kBlocks < NW;
-    constexpr int kPerOperand = kSplitOperands ? 1 : Tile::kBlocks / NW;
+    constexpr int kPerOperand = Tile::kBlocks / NW;
     constexpr int kRowStep = NW * Tile::kRowsPerBlock;
-    static_assert(kRowStep % 16 == 0 && (kSplitOperands ? kBlocksPerWave == 1 && 2 * Tile::kBlocks == NW : 2 * kPerOperand == kBlocksPerWave),
-                  "block assignment");
+    static_assert(kRowStep % 16 == 0 && 2 * kPerOperand == kBlocksPerWave, "block assignment");
     constexpr int kDqSteps = 4 * DB;           // MFMAs of dQ^T per tile
     constexpr int kSteps = kDqSteps + 4 * KK;  // + S^T and dP^T of the next tile
-    constexpr int kRing = (DROPOUT && D == 128) || D == 32 ? 4 : 6;  // (registers; at D = 32 the dQ^T steps are four)
+    constexpr int kRing = DROPOUT && D == 128 ? 4 : 6;  // (registers)
     static_assert(kRing <= kDqSteps, "the vector phase requests dQ fragments only");
     // The workgroup's Q and dO rows reach the registers through LDS as well: lanes own rows, so direct loads
     // touch 32 cache lines per instruction, while LDS-direct loads fetch whole rows. Each wave stages its
@@ -395,16 +392,10 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
 
     // A wave fetches blocks wave, wave + NW, ... of the K tile and of the V tile: their rows are a
     // multiple of 16 apart, so one per-lane source offset serves all of them.
-    const int my_block = kSplitOperands ? wave % Tile::kBlocks : wave;
-    const uint32_t koff = static_cast<uint32_t>(Tile::src_off(my_block, lane, krow_bytes));
-    const uint32_t voff = static_cast<uint32_t>(Tile::src_off(my_block, lane, vrow_bytes));
+    const uint32_t koff = static_cast<uint32_t>(Tile::src_off(wave, lane, krow_bytes));
+    const uint32_t voff = static_cast<uint32_t>(Tile::src_off(wave, lane, vrow_bytes));
     auto issue_tile = [&](int t) {
-        char* stage = smem + (t % kStages) * kStageBytes + my_block * 1024;
-        if constexpr (kSplitOperands) {
-            if (wave < Tile::kBlocks) lds_direct_load16(kbase + static_cast<int64_t>(t) * kBN * krow_bytes, koff, stage);
-            else lds_direct_load16(vbase + static_cast<int64_t>(t) * kBN * vrow_bytes, voff, stage + Tile::kBytes);
-            return;
-        }
+        char* stage = smem + (t % kStages) * kStageBytes + wave * 1024;
 #pragma unroll
         for (int i = 0; i < kPerOperand; ++i)
             lds_direct_load16(kbase + (static_cast<int64_t>(t) * kBN + i * kRowStep) * krow_bytes, koff, stage + i * NW * 1024);
@@ -1720,19 +1711,20 @@ int launch_dq_waves(const KParams& p, hipStream_t stream) {
     return static_cast<int>(hipGetLastError());
 }
 
-// whether the phased dQ kernel serves this problem (no mask, 256-row workgroups; with dropout at D = 128 it fits
-// its registers only under the causal mask and with a fragment ring of 4)
+// whether the phased dQ kernel serves this problem (no mask, 256-row workgroups, D >= 64; with dropout at D = 128 it
+// fits its registers only under the causal mask and with a fragment ring of 4). At D = 32 the kernel above needs 96
+// registers, two of its workgroups share a CU, and that measured 27 % faster than the phased pairs.
 template <int D, int MASK>
 bool dq_is_phased(const KParams& p) {
-    return MASK == kNoMask && p.S % 256 == 0 && (D <= 64 || p.thr8 <= 0 || p.causal);
+    return MASK == kNoMask && D >= 64 && p.S % 256 == 0 && (D == 64 || p.thr8 <= 0 || p.causal);
 }
 
 template <typename T, int D, bool CAUSAL, int MASK>
 int launch_dq_dropout(const KParams& p, hipStream_t stream, bool with_delta) {
-    if constexpr (MASK == kNoMask) {
+    if constexpr (MASK == kNoMask && D >= 64) {
         if (dq_is_phased<D, MASK>(p)) {
             const dim3 grid(p.B * p.H * (p.S / 256)), block(512);
-            if constexpr (D <= 64 || CAUSAL) {
+            if constexpr (D == 64 || CAUSAL) {
                 if (p.thr8 > 0) {
                     if (with_delta) hipLaunchKernelGGL((mfma_dq_phased_kernel<T, D, CAUSAL, true, true>), grid, block, 0, stream, p);
                     else hipLaunchKernelGGL((mfma_dq_phased_kernel<T, D, CAUSAL, true, false>), grid, block, 0, stream, p);

@@ -144,7 +144,7 @@ bool mfma_supported(int which, int dtype, const KParams& p) {
 // The phased dQ kernel (no mask, 256-row workgroups, no dropout at D = 128) can compute delta itself.
 bool mfma_dq_fuses_delta(const KParams& p) {
     if (p.mask != nullptr || p.S % 256 != 0) return false;
-    if (!(p.D <= 64 || p.thr8 <= 0 || p.causal)) return false;  // (the phased dQ kernel's own limits)
+    if (p.D < 64 || !(p.D == 64 || p.thr8 <= 0 || p.causal)) return false;  // (the phased dQ kernel's own limits)
     return aligned16(p.o) && strides8(p.os) && tile_offsets_fit(p.os);
 }
 
