@@ -89,6 +89,10 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
     float lse = p.lse[static_cast<int64_t>(bh) * p.S + qrow_ld];
     const float dlt = p.delta[static_cast<int64_t>(bh) * p.S + qrow_ld];
     const float c = p.scale_log2;
+    // Without dropout (and where the registers allow) the subtraction in dS = P (dP - delta) is left to the matrix pipe:
+    // the dP^T accumulators start from delta and take the product with the dO rows negated, which gives delta - dP^T;
+    // dS^T then comes out negated and the sign goes into the scale of the final store.
+    constexpr bool kDeltaInAcc = !DROPOUT && !DMASK && D <= 64;
 
     f32x16 acc[DB];
 #pragma unroll
@@ -163,6 +167,16 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
     }
     settle(lse);
     settle(dlt);
+    f32x16 dlt16;
+    if constexpr (kDeltaInAcc) {
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) gf[kk][i] ^= 0x80008000u;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dlt16[i] = dlt;
+        asm volatile("" : "+v"(dlt16));  // (kept in registers: as a splat it would be made anew for every block)
+    }
 
     const int row_off0 = Tile::off(l32, h);
     const int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
@@ -231,6 +245,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
             for (int kk = 0; kk < KK; ++kk) fr[kk] = lds_read16(sK, (row_off0 ^ (kk << 5)) + 32 * kb * Tile::kRowBytes);
             __builtin_amdgcn_sched_barrier(0);
             f32x16 st = zero16(), dpt = zero16();
+            if constexpr (kDeltaInAcc) dpt = dlt16;
 #pragma unroll
             for (int kk = 0; kk < KK; ++kk) {
                 st = Mma<T>::run(fr[kk], qf[kk], st);
@@ -275,7 +290,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
                     }
             }
 #pragma unroll
-            for (int i = 0; i < 16; ++i) ds[i] *= dpt[i] - dlt;
+            for (int i = 0; i < 16; ++i) ds[i] *= kDeltaInAcc ? dpt[i] : dpt[i] - dlt;
             if constexpr (DMASK) {
                 const int64_t at = b * p.dms[0] + hd * p.dms[1] + static_cast<int64_t>(qrow) * p.dms[2] + t0 + 32 * kb + 4 * h;
                 if (p.dmask_acc) {
@@ -308,7 +323,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
         using Store = RowBlockStore<T, DB>;
         static_assert(NW * Store::kPatchBytes <= kStages * kStageBytes, "patches must fit into the ring");
         char* out0 = static_cast<char*>(p.dq) + (b * p.dqs[0] + hd * p.dqs[1] + static_cast<int64_t>(wrow0) * p.dqs[2]) * 2;
-        const float sc = p.scale;
+        const float sc = kDeltaInAcc ? -p.scale : p.scale;
         Store::run(acc, [sc](float x) { return x * sc; }, smem + wave * Store::kPatchBytes, out0, p.dqs[2] * 2, lane,
                    RAGGED ? p.S - wrow0 : 32);
     }
@@ -642,6 +657,10 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
         vf[kk] = *reinterpret_cast<const u32x4*>(vbase + static_cast<int64_t>(key_ld) * p.vs[2] * 2 + (2 * kk + h) * 16);
     }
     const float c = p.scale_log2;
+    // Without dropout the subtraction in dS = P (dP - delta) is left to the matrix pipe: the dP accumulators start from
+    // the rows' delta values (as they come from the tile: the accumulator's layout) and take the product with the V
+    // fragments negated, which gives delta - dP; dS then comes out negated and the sign goes into dK's final scale.
+    constexpr bool kDeltaInAcc = !DROPOUT;
 
     f32x16 dk[DB], dv[DB];
 #pragma unroll
@@ -725,6 +744,10 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
     for (int kk = 0; kk < KK; ++kk) {
         settle(kf[kk]);
         settle(vf[kk]);
+        if constexpr (kDeltaInAcc) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) vf[kk][i] ^= 0x80008000u;
+        }
     }
 
     const int row_off0 = Tile::off(l32, h);
@@ -791,6 +814,13 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
             for (int kk = 0; kk < KK; ++kk) fr[kk] = lds_read16(sQ, (row_off0 ^ (kk << 5)) + qoff);
             __builtin_amdgcn_sched_barrier(0);
             f32x16 s = zero16(), dp = zero16();
+            if constexpr (kDeltaInAcc) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const f32x4 d4 = *reinterpret_cast<const f32x4*>(sDelta + 32 * qb + 8 * g + 4 * h);
+                    dp[4 * g + 0] = d4.x; dp[4 * g + 1] = d4.y; dp[4 * g + 2] = d4.z; dp[4 * g + 3] = d4.w;
+                }
+            }
 #pragma unroll
             for (int kk = 0; kk < KK; ++kk) {
                 s = Mma<T>::run(fr[kk], kf[kk], s);
@@ -833,7 +863,8 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
                 if constexpr (DROPOUT) mine = dropout_block(p, bh, (rb + 8 * (lane & 3) + 4 * h) >> 2, key >> 2);
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    const f32x4 d4 = *reinterpret_cast<const f32x4*>(sDelta + 32 * qb + 8 * g + 4 * h);
+                    f32x4 d4 = {0.f, 0.f, 0.f, 0.f};
+                    if constexpr (!kDeltaInAcc) d4 = *reinterpret_cast<const f32x4*>(sDelta + 32 * qb + 8 * g + 4 * h);
                     uint32_t dw[4];
                     if constexpr (DROPOUT) {
                         const Philox4 r = quad_bcast_from(g, mine);  // lane g of the quad generated rows rb + 8 g + 4 h .. +3
@@ -852,7 +883,7 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
                         } else {
                             pr[i] = pv;
                         }
-                        ds[i] = pv * (dpv - d4[bb]);
+                        ds[i] = kDeltaInAcc ? pv * dpv : pv * (dpv - d4[bb]);
                     }
                 }
 #pragma unroll
@@ -888,7 +919,7 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
         char* patch = smem + wave * Store::kPatchBytes;
         char* dk0 = static_cast<char*>(p.dk) + (b * p.dks[0] + hd * p.dks[1] + static_cast<int64_t>(wkey0) * p.dks[2]) * 2;
         char* dv0 = static_cast<char*>(p.dv) + (b * p.dvs[0] + hd * p.dvs[1] + static_cast<int64_t>(wkey0) * p.dvs[2]) * 2;
-        const float sc = p.scale;
+        const float sc = kDeltaInAcc ? -p.scale : p.scale;
         const int keys_here = RAGGED ? p.S - wkey0 : 32;
         Store::run(dk, [sc](float x) { return x * sc; }, patch, dk0, p.dks[2] * 2, lane, keys_here);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // patch read before it is rewritten
