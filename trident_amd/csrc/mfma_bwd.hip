@@ -355,7 +355,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
     static_assert(kRowStep % 16 == 0 && 2 * kPerOperand == kBlocksPerWave, "block assignment");
     constexpr int kDqSteps = 4 * DB;           // MFMAs of dQ^T per tile
     constexpr int kSteps = kDqSteps + 4 * KK;  // + S^T and dP^T of the next tile
-    constexpr int kRing = DROPOUT && D == 128 ? 4 : 6;  // (registers)
+    constexpr int kRing = D == 128 ? 4 : 6;  // (registers: with dropout the Philox state, without it the delta accumulators)
     static_assert(kRing <= kDqSteps, "the vector phase requests dQ fragments only");
     // The workgroup's Q and dO rows reach the registers through LDS as well: lanes own rows, so direct loads
     // touch 32 cache lines per instruction, while LDS-direct loads fetch whole rows. Each wave stages its
@@ -457,6 +457,20 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
         if (h == 0) p.delta[static_cast<int64_t>(bh) * p.S + qrow] = dlt;
     }
 
+    // Without dropout the subtraction in dS = P (dP - delta) is left to the matrix pipe: the dP^T accumulators start from
+    // delta and take the product with the dO rows negated (delta - dP^T); dS^T comes out negated and the sign goes into
+    // the scale of the final store.
+    constexpr bool kDeltaInAcc = !DROPOUT;
+    f32x16 dlt16;
+    if constexpr (kDeltaInAcc) {
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) gf[kk][i] ^= 0x80008000u;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dlt16[i] = dlt;
+        asm volatile("" : "+v"(dlt16));  // (kept in registers: as a splat it would be made anew for every tile)
+    }
     const int tr_off0 = Tile::tr_off(0, 0, lane), tr_off1 = Tile::tr_off(0, 1, lane);
 
     // fragment n of the matrix phase of tile t: n < kDqSteps: K^T of tile t (column block n % DB, K-step
@@ -476,6 +490,10 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
     auto matrix_phase = [&](auto with_dq, int t, bool with_scores = true) {
         constexpr int first = decltype(with_dq)::value ? 0 : kDqSteps;
         f32x16 s_new[2] = {zero16(), zero16()}, dp_new[2] = {zero16(), zero16()};
+        if constexpr (kDeltaInAcc) {
+            dp_new[0] = dlt16;
+            dp_new[1] = dlt16;
+        }
 #pragma unroll
         for (int n = first; n < kSteps; ++n) {
             if (n >= kDqSteps && !with_scores) break;
@@ -546,7 +564,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
                     }
             }
 #pragma unroll
-            for (int i = 0; i < 16; ++i) ds[i] *= dpv[i] - dlt;
+            for (int i = 0; i < 16; ++i) ds[i] *= kDeltaInAcc ? dpv[i] : dpv[i] - dlt;
             bop[2 * kb + 0] = pack8<T>(&ds[0]);
             bop[2 * kb + 1] = pack8<T>(&ds[8]);
         };
@@ -590,7 +608,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
         using Store = RowBlockStore<T, DB>;
         static_assert(NW * Store::kPatchBytes <= kStages * kStageBytes, "patches must fit into the ring");
         char* out0 = static_cast<char*>(p.dq) + (b * p.dqs[0] + hd * p.dqs[1] + static_cast<int64_t>(wrow0) * p.dqs[2]) * 2;
-        const float sc = p.scale;
+        const float sc = kDeltaInAcc ? -p.scale : p.scale;
         // the lane index taken afresh: the epilogue's per-lane offsets are then computed here instead of being
         // kept (or, with every register in use, spilled) across the loop
         int elane = threadIdx.x & 63;
