@@ -129,6 +129,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     float m, l;  // reference exponent (log2 domain, scaled) and this lane's partial sum
     float m_use;  // m, or 0 while no key has been seen (m = -inf): what the exponents are taken against; follows m
     const float c = p.scale_log2;
+    const float inv_scale = 1.f / p.scale;  // (a mask value joins its score before the scale: s + mask / scale)
 
     char* mask_lds = smem + kStages * kStageBytes + wave * kMaskBytes;
     auto issue_mask = [&](int t) {  // mask block of tile t -> this wave's region (8 LDS-direct loads), unless it is all zero
@@ -277,7 +278,6 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     constexpr bool kDefer = !DROPOUT;
     float xd[16];        // deferred exponents and then probabilities
     float m_def = 0.f;   // the reference exponent they are taken against
-    float c_def = c;     // the factor they are still to be multiplied by (1 where the mask has been added: scaled already)
     const uint32_t one2 = Mma<T>::pack2(1.f, 1.f);
     u32x4 ones = {one2, one2, one2, one2};
     asm volatile("" : "+v"(ones));  // (kept in registers: as a constant it would be made anew from scalars in every tile)
@@ -322,8 +322,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
                     for (int e = 0; e < 8; ++e)
                         if (e * ne / 8 == ls) {
                             float& v = xd[8 * (g - 2) + e];
-                            if constexpr (MASK == kNoMask) v = fast_exp2(fmaf(v, c, -m_def));
-                            else v = fast_exp2(fmaf(v, c_def, -m_def));
+                            v = fast_exp2(fmaf(v, c, -m_def));
                         }
                     if (ls == pack_step) pb[g] = pack8<T>(&xd[8 * (g - 2)]);
                 }
@@ -382,14 +381,12 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
                 x[i] = sc[0][i];
                 x[16 + i] = sc[1][i];
             }
-            // scores in the log2 domain; without a mask - and in a tile whose mask is all zero - the scale is folded into
-            // the exponent's multiply-add (cc: the factor still to apply)
-            float cc = c;
+            // The scale (to the log2 domain) is folded into the exponent's multiply-add; a mask value is added before it,
+            // divided by the scale: one multiply-add per score, none in a tile whose mask is all zero.
             if constexpr (MASK != kNoMask) {
                 if (!mask_is_zero(j)) {
 #pragma unroll
-                    for (int e = 0; e < 32; ++e) x[e] = fmaf(mk[e], kLog2e, x[e] * c);
-                    cc = 1.f;
+                    for (int e = 0; e < 32; ++e) x[e] = fmaf(mk[e], inv_scale, x[e]);
                 }
             }
             if (CAUSAL && t0 + kBN - 1 > wrow0) {
@@ -415,7 +412,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
                 mx1 = max3(mx1, x[16 + e], x[17 + e]);
             }
             mx = max_xor32(max3(mx, x[15], max3(mx1, x[31], x[31])));
-            mx *= cc;
+            mx *= c;
             // Lazy rescaling: m is the reference exponent of l and of the O accumulators, not
             // necessarily the running maximum. It is only moved (and O rescaled) when some row of
             // the wave outgrew it by more than 2^kTau; until then probabilities may exceed 1 by
@@ -444,8 +441,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
             for (int ks = 0; ks < kNow; ++ks) {
 #pragma unroll
                 for (int e = 8 * ks; e < 8 * ks + 8; ++e) {
-                    if constexpr (MASK == kNoMask) x[e] = fast_exp2(fmaf(x[e], c, -m_use));
-                    else x[e] = fast_exp2(fmaf(x[e], cc, -m_use));
+                    x[e] = fast_exp2(fmaf(x[e], c, -m_use));
                 }
                 if constexpr (!DROPOUT) pb[ks] = pack8<T>(&x[8 * ks]);
                 if (ks < 2 && issued) issue_slice(j + dist, 2 + ks);
@@ -459,7 +455,6 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) xd[e] = x[16 + e];
                 m_def = m_use;
-                c_def = cc;
             }
             if constexpr (DROPOUT) {
                 // row sum before dropping, in fp32: four interleaved partial sums (a dependent add waits
