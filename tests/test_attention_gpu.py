@@ -523,7 +523,7 @@ def test_more_items_than_compute_units(batches, heads, S, D, variant, device):
 
 
 @pytest.mark.parametrize("B,H,S,D,causal", [(8, 16, 896, 32, False), (8, 16, 2176, 32, True), (8, 16, 1024, 32, True),
-                                            (6, 16, 1152, 64, True)])
+                                            (6, 16, 1152, 64, True), (8, 12, 896, 32, "mask"), (8, 12, 640, 64, "mask")])
 def test_a_head_does_not_depend_on_its_company(B, H, S, D, causal, device):
     """Several workgroups resident per compute unit (small heads: four 4-wave workgroups): every head of a launch with a
     thousand workgroups gets bit for bit what it gets in a launch of its batch alone, and two heads match the oracle.
@@ -534,16 +534,22 @@ def test_a_head_does_not_depend_on_its_company(B, H, S, D, causal, device):
     q, k, v, d_o = _gen((B, H, S, D), 4100 + S + D, dtype)
     scale = 1.0 / math.sqrt(D)
     tq, tk, tv, tdo = [x.to(device) for x in (q, k, v, d_o)]
-    o, lse = Attention._forward(tq, tk, tv, None, 0.0, causal, scale, 0, 0)
-    dq, dk, dv, _ = Attention._backward(tdo, tq, tk, tv, o, lse, None, scale, 0.0, causal, 0, 0, False)
+    mask = tm = None
+    if causal == "mask":  # (a dense fp32 mask shared by the heads of a batch)
+        causal = False
+        mask = torch.randn(B, 1, S, S, generator=torch.Generator().manual_seed(4099))
+        tm = mask.to(device)
+    o, lse = Attention._forward(tq, tk, tv, tm, 0.0, causal, scale, 0, 0)
+    dq, dk, dv, _ = Attention._backward(tdo, tq, tk, tv, o, lse, tm, scale, 0.0, causal, 0, 0, False)
     for b in range(B):
         sl = slice(b, b + 1)
-        o1, lse1 = Attention._forward(tq[sl], tk[sl], tv[sl], None, 0.0, causal, scale, 0, 0)
-        dq1, dk1, dv1, _ = Attention._backward(tdo[sl], tq[sl], tk[sl], tv[sl], o1, lse1, None, scale, 0.0, causal, 0, 0, False)
+        m1 = None if tm is None else tm[sl]
+        o1, lse1 = Attention._forward(tq[sl], tk[sl], tv[sl], m1, 0.0, causal, scale, 0, 0)
+        dq1, dk1, dv1, _ = Attention._backward(tdo[sl], tq[sl], tk[sl], tv[sl], o1, lse1, m1, scale, 0.0, causal, 0, 0, False)
         for name, whole, part in (("O", o, o1), ("LSE", lse, lse1), ("dQ", dq, dq1), ("dK", dk, dk1), ("dV", dv, dv1)):
             assert torch.equal(whole[sl], part), f"{name} of batch {b} differs between the launches"
     hs = slice(H - 2, H)
-    kw = dict(is_causal=causal, scale=scale)
+    kw = dict(is_causal=causal, scale=scale, mask=None if mask is None else mask[B - 1:])
     qs, ks, vs, gs = [x[B - 1:, hs] for x in (q, k, v, d_o)]
     o_ref, _ = parity.oracle_forward(qs, ks, vs, **kw)
     parity.close(o[B - 1:, hs], o_ref, dtype, "company O")
