@@ -117,6 +117,7 @@ int make_params(const TriAttnArgs* a, int need, KParams* p) {
     p->mask_dtype = a->mask_dtype;
     p->scale = a->softmax_scale;
     p->scale_log2 = a->softmax_scale * kLog2e;
+    p->inv_scale = a->softmax_scale != 0.f ? 1.f / a->softmax_scale : 0.f;
     p->seed_lo = static_cast<uint32_t>(a->seed);
     p->seed_hi = static_cast<uint32_t>(a->seed >> 32);
     p->offset = static_cast<uint32_t>(a->offset);

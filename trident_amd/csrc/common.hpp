@@ -35,6 +35,7 @@ struct KParams {
     int mask_dtype;
     float scale;       // softmax_scale
     float scale_log2;  // softmax_scale * log2(e)
+    float inv_scale;   // 1 / softmax_scale (0 where the scale is 0)
     uint32_t seed_lo, seed_hi, offset;
     int dmask_acc;     // dmask is summed over a broadcast dimension (stride 0): fp32 buffer, atomic adds
     int thr8;          // 0 = no dropout; keep iff u8 >= thr8

@@ -89,7 +89,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
     float lse = p.lse[static_cast<int64_t>(bh) * p.S + qrow_ld];
     const float dlt = p.delta[static_cast<int64_t>(bh) * p.S + qrow_ld];
     const float c = p.scale_log2;
-    [[maybe_unused]] const float inv_scale = 1.f / p.scale;  // (a mask value joins its score before the scale: s + mask / scale)
+    [[maybe_unused]] const float inv_scale = p.inv_scale;  // (a mask value joins its score before the scale: s + mask / scale)
     // Without dropout (and where the registers allow) the subtraction in dS = P (dP - delta) is left to the matrix pipe:
     // the dP^T accumulators start from delta and take the product with the dO rows negated, which gives delta - dP^T;
     // dS^T then comes out negated and the sign goes into the scale of the final store.
@@ -398,7 +398,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dq_phased_kernel(const KParams p)
     for (int blk = 0; blk < kRowLoads; ++blk)
         lds_direct_load16(gorows, static_cast<uint32_t>(Tile::src_off(blk, lane, p.dos[2] * 2)), g_stage + blk * 1024);
     const float c = p.scale_log2;
-    [[maybe_unused]] const float inv_scale = 1.f / p.scale;  // (a mask value joins its score before the scale: s + mask / scale)
+    [[maybe_unused]] const float inv_scale = p.inv_scale;  // (a mask value joins its score before the scale: s + mask / scale)
 
     f32x16 acc[DB];
 #pragma unroll
@@ -677,7 +677,7 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
         vf[kk] = *reinterpret_cast<const u32x4*>(vbase + static_cast<int64_t>(key_ld) * p.vs[2] * 2 + (2 * kk + h) * 16);
     }
     const float c = p.scale_log2;
-    [[maybe_unused]] const float inv_scale = 1.f / p.scale;  // (a mask value joins its score before the scale: s + mask / scale)
+    [[maybe_unused]] const float inv_scale = p.inv_scale;  // (a mask value joins its score before the scale: s + mask / scale)
     // Without dropout the subtraction in dS = P (dP - delta) is left to the matrix pipe: the dP accumulators start from
     // the rows' delta values (as they come from the tile: the accumulator's layout) and take the product with the V
     // fragments negated, which gives delta - dP; dS then comes out negated and the sign goes into dK's final scale.
@@ -994,7 +994,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
     const float* delta_base = p.delta + static_cast<int64_t>(bh) * p.S;
 
     const float c = p.scale_log2;
-    [[maybe_unused]] const float inv_scale = 1.f / p.scale;  // (a mask value joins its score before the scale: s + mask / scale)
+    [[maybe_unused]] const float inv_scale = p.inv_scale;  // (a mask value joins its score before the scale: s + mask / scale)
 
     f32x16 dk[DH], dv[DH];
 #pragma unroll
@@ -1396,7 +1396,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
     const float* lse_base = p.lse + static_cast<int64_t>(bh) * p.S;
     const float* delta_base = p.delta + static_cast<int64_t>(bh) * p.S;
     const float c = p.scale_log2;
-    [[maybe_unused]] const float inv_scale = 1.f / p.scale;  // (a mask value joins its score before the scale: s + mask / scale)
+    [[maybe_unused]] const float inv_scale = p.inv_scale;  // (a mask value joins its score before the scale: s + mask / scale)
     float key_bias = 0.f;  // mask value of this lane's key, log2 domain
     if constexpr (KEYMASK != kNoMask) key_bias = mask_at<T, KEYMASK>(p.mask, b * p.ms[0] + hd * p.ms[1] + key) * kLog2e;
 

@@ -28,7 +28,6 @@ namespace tri {
 namespace {
 
 constexpr int kBN = 64;      // keys per tile
-constexpr int kStages = 4;   // LDS ring depth
 constexpr float kTau = 8.f;  // lazy-rescale threshold, log2 domain
 
 enum MaskKind { kNoMask = 0, kMaskF32 = 1, kMaskT = 2 };
@@ -39,6 +38,13 @@ template <typename T, int D, int NW, bool CAUSAL, int MASK, bool DROPOUT, bool R
 __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     static_assert(!RAGGED || (NW == 4 && MASK == 0), "ragged lengths: 4 waves, no mask");
     using Tile = SwzTile<D>;
+    // An fp32 mask at D = 128 (8 waves, no dropout) needs 64 KiB of LDS for its staging regions. The ring then has
+    // three slots per operand and the K tiles run one tile ahead of the V tiles: K of tile t is last read one matrix
+    // phase before V of tile t, so with K(j + dist) and V(j + dist - 1) requested together every tile keeps the lead
+    // it has in the ring of four, and both fit three slots.
+    constexpr bool kLeadK = D == 128 && MASK == 1 && NW == 8 && !DROPOUT;
+    constexpr int kStages = kLeadK ? 3 : 4;  // LDS ring depth
+    constexpr int kLag = kLeadK ? 1 : 0;     // how many tiles the V requests trail the K requests
     constexpr int kBM = 32 * NW;
     constexpr int kKBytes = Tile::kBytes;
     constexpr int kStageBytes = 2 * Tile::kBytes;  // K tile, V tile
@@ -61,7 +67,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     // for one of the operand type) when it fits (D = 64): lanes own rows, so direct loads would touch 32 cache
     // lines per instruction, while LDS-direct loads fetch whole rows (256 or 128 bytes) and the swizzled tile is
     // read back 16 or 8 bytes at a time. The region has the geometry of a 32-row SwzTile<128> / SwzTile<64>.
-    constexpr bool kMaskViaLds = MASK != kNoMask && (D <= 64 || (MASK == kMaskT && NW == 8 && !DROPOUT));  // (D = 128: 4 KiB regions fit, 8 KiB ones do not; with dropout the registers for the staged values are not there)
+    constexpr bool kMaskViaLds = MASK != kNoMask && (D <= 64 || (NW == 8 && !DROPOUT));  // (D = 128: 4 KiB regions fit, 8 KiB ones do not; with dropout the registers for the staged values are not there)
     constexpr int kMaskElt = MASK == kMaskF32 ? 4 : 2;
     using MaskTile = std::conditional_t<MASK == kMaskF32, SwzTile<128>, SwzTile<64>>;
     constexpr int kMaskBytes = 32 * MaskTile::kRowBytes;
@@ -129,7 +135,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     float m, l;  // reference exponent (log2 domain, scaled) and this lane's partial sum
     float m_use;  // m, or 0 while no key has been seen (m = -inf): what the exponents are taken against; follows m
     const float c = p.scale_log2;
-    const float inv_scale = 1.f / p.scale;  // (a mask value joins its score before the scale: s + mask / scale)
+    const float inv_scale = p.inv_scale;  // (a mask value joins its score before the scale: s + mask / scale)
 
     char* mask_lds = smem + kStages * kStageBytes + wave * kMaskBytes;
     auto issue_mask = [&](int t) {  // mask block of tile t -> this wave's region (8 LDS-direct loads), unless it is all zero
@@ -154,8 +160,10 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     static_assert(kPerOperand >= 1 && kRowStep % 16 == 0 && 2 * kPerOperand == kBlocksPerWave, "block assignment");  // (D = 32: 4 waves)
     const uint32_t koff = static_cast<uint32_t>(Tile::src_off(wave, lane, krow_bytes));
     const uint32_t voff = static_cast<uint32_t>(Tile::src_off(wave, lane, vrow_bytes));
-    // load number idx (0 .. kBlocksPerWave-1) of this wave's share of tile t -> ring slot t % kStages
-    auto issue_load = [&](int t, int idx) {
+    // load number idx (0 .. kBlocksPerWave-1) of this wave's share of the K tile t (the first kPerOperand) and of the V
+    // tile t - kLag (the others) -> ring slot (tile % kStages) of the operand
+    auto issue_load = [&](int tk, int idx) {
+        const int t = idx < kPerOperand ? tk : tk - kLag;
         char* stage = smem + (t % kStages) * kKBytes + wave * 1024;
         const int i = idx % kPerOperand;
         if (RAGGED && (t + 1) * kBN > p.S) {  // the sequence ends inside this tile: clamped rows, offsets from the tile's first row
@@ -174,14 +182,15 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     // The loads of a tile are issued in four slices spread over the softmax phase: a wave stalls on a
     // load until the memory pipeline accepts it, and sixteen loads arriving at once from the four
     // waves of a group queue up for hundreds of cycles.
-    auto issue_slice = [&](int t, int part) {
+    // (k_ok / v_ok: the K tile t / the V tile t - kLag exists)
+    auto issue_slice = [&](int t, int part, bool k_ok = true, bool v_ok = true) {
 #pragma unroll
         for (int idx = 0; idx < kBlocksPerWave; ++idx)
-            if (idx % 4 == part) issue_load(t, idx);
+            if (idx % 4 == part && (idx < kPerOperand ? k_ok : v_ok)) issue_load(t, idx);
     };
-    auto issue_tile = [&](int t) {
+    auto issue_tile = [&](int t, bool k_ok = true, bool v_ok = true) {
 #pragma unroll
-        for (int part = 0; part < 4; ++part) issue_slice(t, part);
+        for (int part = 0; part < 4; ++part) issue_slice(t, part, k_ok, v_ok);
     };
     // Ping-pong schedule (8 waves): waves w and w+4 share a SIMD. The loop alternates a softmax
     // phase (vector ALU only) and a matrix phase (P V of this tile, then S^T of the next), with a
@@ -191,19 +200,25 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     constexpr bool kPingPong = NW == 8;
     const int group = kPingPong ? wave >> 2 : 0;
     const int dist = 2 + group;
-    auto wait_loads = [&](bool mask_block, bool tile) {  // all but the youngest (mask block, tile) have landed
+    // all but the youngest (mask block, tile requests: of both operands, of the V tile only, none) have landed
+    auto wait_loads = [&](bool mask_block, bool tile, bool tile_v = false) {
         constexpr int kM = kMaskBytes / 1024, kB = kBlocksPerWave;
         if (mask_block && tile) TRI_WAIT_VMCNT(kM + kB);
+        else if (mask_block && kLeadK && tile_v) TRI_WAIT_VMCNT(kM + kPerOperand);
         else if (mask_block) TRI_WAIT_VMCNT(kM);
         else if (tile) TRI_WAIT_VMCNT(kB);
+        else if (kLeadK && tile_v) TRI_WAIT_VMCNT(kPerOperand);
         else TRI_WAIT_VMCNT(0);
     };
     int n_first;
     auto request_first_tiles = [&]() {  // (the Q rows were requested before, so both latencies overlap)
-        n_first = min(dist, n_tiles);
-        issue_tile(0);
-        if (n_first > 1) issue_tile(1);
-        if (n_first > 2) issue_tile(2);
+        n_first = min(dist, n_tiles);                    // K tiles 0 .. n_first - 1
+        const int v_first = min(dist - kLag, n_tiles);   // V tiles 0 .. v_first - 1
+#pragma unroll
+        for (int t = 0; t < 3; ++t) {
+            const bool k_ok = t < n_first, v_ok = t - kLag >= 0 && t - kLag < v_first;
+            if (k_ok || v_ok) issue_tile(t, k_ok, v_ok);
+        }
     };
     request_first_tiles();
 
@@ -237,12 +252,12 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
         }
     };
     // mask block t from this wave's LDS region, then the request for block t+1
-    auto take_mask_block = [&](int t, bool first, bool tile_in_flight) {
+    auto take_mask_block = [&](int t, bool first, bool tile_in_flight, bool v_in_flight = false) {
         if constexpr (kMaskViaLds) {
             // block t was requested a matrix phase ago and only the newest tile load may be younger
             // (block 0 precedes tile 0, which has landed)
             if (!mask_is_zero(t)) {
-                if (!first) wait_loads(false, tile_in_flight);
+                if (!first) wait_loads(false, tile_in_flight, v_in_flight);
 #pragma unroll
                 for (int g = 0; g < 8; ++g) {  // keys 32 (g / 4) + 8 (g % 4) + 4 h .. + 3 of this lane's row
                     if constexpr (MASK == kMaskF32) {
@@ -344,14 +359,14 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     l = 0.f;
     // tile 0 has landed and is visible to all waves (a later item's requests are older than the stores of the
     // item before it: everything is awaited)
-    if (!first_item) TRI_WAIT_VMCNT(0);
+    if (!first_item || kLeadK) TRI_WAIT_VMCNT(0);  // (the K-leading ring requests in another order: it awaits everything)
     else if (n_first == 3) TRI_WAIT_VMCNT(2 * kBlocksPerWave);
     else if (n_first == 2) TRI_WAIT_VMCNT(kBlocksPerWave);
     else TRI_WAIT_VMCNT(0);
     lds_barrier();
     if (kPingPong && group == 1) {
         // group 1 starts one phase late; group 0 reads tile 1 in its first matrix phase
-        if (first_item && n_first == 3) TRI_WAIT_VMCNT(kBlocksPerWave);
+        if (first_item && n_first == 3 && !kLeadK) TRI_WAIT_VMCNT(kBlocksPerWave);
         else TRI_WAIT_VMCNT(0);
         lds_barrier();
     }
@@ -369,8 +384,9 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     // One step of the tile loop; st = j % kStages is a literal at each of the loop's four calls.
     auto tile_step = [&](const int j, const int st) __attribute__((always_inline)) {
         // slot of tile j+dist: every wave is done with the tile it held (two barriers ago at the latest)
-        const bool issued = j + dist < n_tiles;
-        if (issued) issue_slice(j + dist, 0);
+        const bool issued = j + dist < n_tiles;            // the K tile requested in this step exists
+        const bool issued_v = j + dist - kLag < n_tiles;   // ... its V tile (the same tile, or the one before it)
+        if (issued_v) issue_slice(j + dist, 0, issued, issued_v);
         const int t0 = j * kBN;
         constexpr bool active = true;
 
@@ -435,7 +451,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
             // exponentials in four groups of eight keys (one B operand each); the remaining loads of the
             // next tile and the first fragment reads of the matrix phase (tile j has been visible since
             // the previous barrier) are issued between the groups, so that none of them queues
-            if (issued) issue_slice(j + dist, 1);
+            if (issued_v) issue_slice(j + dist, 1, issued, issued_v);
             constexpr int kNow = kDefer ? 2 : 4;  // groups whose exponentials are taken here
 #pragma unroll
             for (int ks = 0; ks < kNow; ++ks) {
@@ -444,7 +460,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
                     x[e] = fast_exp2(fmaf(x[e], c, -m_use));
                 }
                 if constexpr (!DROPOUT) pb[ks] = pack8<T>(&x[8 * ks]);
-                if (ks < 2 && issued) issue_slice(j + dist, 2 + ks);
+                if (ks < 2 && issued_v) issue_slice(j + dist, 2 + ks, issued, issued_v);
                 if (ks < 2) {
 #pragma unroll
                     for (int r = kRing / 2 * ks; r < kRing / 2 * (ks + 1); ++r) ring[r] = frag(Yes{}, st, r);
@@ -493,7 +509,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
         // after the barrier it is visible to every wave, and the partner group changes phase. The
         // fragment reads stay in flight across the barrier: nothing overwrites their slot before the
         // barrier after next.
-        wait_loads(kMaskViaLds && with_s && !mask_is_zero(j + 1), issued);
+        wait_loads(kMaskViaLds && with_s && !mask_is_zero(j + 1), issued, issued_v);
         __builtin_amdgcn_sched_barrier(0);
         asm volatile("s_barrier" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
@@ -508,7 +524,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
             __builtin_amdgcn_s_setprio(2);
             matrix_phase(Yes{}, Yes{}, st, with_s || DROPOUT);
             __builtin_amdgcn_s_setprio(0);
-            if (with_s) take_mask_block(j + 1, false, issued);
+            if (with_s) take_mask_block(j + 1, false, issued, issued_v);
         }
         if constexpr (kPingPong) {
             __builtin_amdgcn_sched_barrier(0);
@@ -516,11 +532,17 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    static_assert(kStages == 4, "the tile loop is unrolled over the ring's slots");
+    static_assert(kStages == 4 || kStages == 3, "the tile loop is unrolled over the ring's slots");
     // (a mask and dropout together at D = 128 have no registers to spare for four copies of the step: rolled, the slot
     // is a run-time value there and every fragment read adds it to its address)
     constexpr bool kUnrolled = !(D == 128 && MASK != kNoMask && DROPOUT);
-    if constexpr (kUnrolled) {
+    if constexpr (kUnrolled && kStages == 3) {
+        for (int j = 0; j < my_tiles; j += 3) {
+            tile_step(j, 0);
+            if (j + 1 < my_tiles) tile_step(j + 1, 1);
+            if (j + 2 < my_tiles) tile_step(j + 2, 2);
+        }
+    } else if constexpr (kUnrolled) {
         for (int j = 0; j < my_tiles; j += 4) {
             tile_step(j, 0);
             if (j + 1 < my_tiles) tile_step(j + 1, 1);
@@ -531,9 +553,9 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
         for (int j = 0; j < my_tiles; ++j) tile_step(j, j % kStages);
     }
     for (int j = my_tiles; j < n_tiles; ++j) {
-        const bool issued = j + dist < n_tiles;
-        if (issued) issue_tile(j + dist);
-        wait_loads(false, issued);
+        const bool issued = j + dist < n_tiles, issued_v = j + dist - kLag < n_tiles;
+        if (issued_v) issue_tile(j + dist, issued, issued_v);
+        wait_loads(false, issued, issued_v);
         lds_barrier();
         if constexpr (kPingPong) lds_barrier();
     }
