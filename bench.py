@@ -233,11 +233,12 @@ def cpu_baseline(w, reps=3):
 
 
 def config_figures(dev, with_cpu):
-    """Forward and forward+backward figures of all five configurations (each with its own CPU baseline)."""
+    """Forward and forward+backward figures of all five configurations (each with its own CPU baseline) and of the two
+    extra workloads (C3's shape in fp32, a 16-bit problem with head size 32; no CPU baseline)."""
     from trident_amd import workloads
 
     out = {}
-    for name, wl in workloads.WORKLOADS.items():
+    for name, wl in {**workloads.WORKLOADS, **workloads.EXTRA_WORKLOADS}.items():
         pth = Path(wl, dev)
         # (enough warm-up steps for the clock to settle after the idle time of the CPU baseline before it)
         ms, pk = run_steps(pth, 5 if name == "C5" else 30, 2 if name == "C5" else 8)
@@ -261,7 +262,7 @@ def config_figures(dev, with_cpu):
             row["masked_key_fraction"] = round(1.0 - float(lengths.float().mean()) / S, 4)
             row["mask_stream"]["note"] = ("fp32 mask bytes every workgroup asks for (logical: B*H*S*S*4; unique: "
                                           "B*S*S*4, the heads of a batch share it) / kernel duration; HBM peak 8000 GB/s")
-        if with_cpu:
+        if with_cpu and name in workloads.WORKLOADS:
             cb = cpu_baseline(wl, reps={"C3": 1, "C4": 1, "C5": 0}.get(name, 3))
             row.update(cpu_tflops=cb["value"], cpu_cores=cb["cores"])
         out[name] = row
