@@ -183,10 +183,10 @@ int64_t tri_attn_mask_classes_size(const TriAttnArgs* args);
 
 /* Which kernel family a call would run, without launching anything (no counterpart in the reference): pass 0 =
  * tri_attn_fwd, 1 = tri_attn_bwd_dkdv, 2 = tri_attn_bwd_dq on these arguments. Returns 1 for the 16-bit matrix-core
- * (MFMA) kernels (fp16/bf16, D in {64,128}, 16-byte aligned rows; any S without a mask, S a multiple of 128 with
+ * (MFMA) kernels (fp16/bf16, D in {32,64,128}, 16-byte aligned rows; any S without a mask, S a multiple of 128 with
  * one); 2 for the 32-row-tile matrix-core kernels (everything else whose pointers and strides are multiples of
- * four elements: fp32 problems on the fp32 matrix instruction with fp32 products and sums; fp16/bf16 problems with D in
- * {16,32} or masked lengths that are no multiple of 128 on the 16-bit 32x32x8 instruction);
+ * four elements: fp32 problems on the fp32 matrix instruction with fp32 products and sums; fp16/bf16 problems with
+ * D = 16 or masked lengths that are no multiple of 128 on the 16-bit 32x32x8 instruction);
  * 0 for the general vector-ALU kernels (views that are not aligned so); or a negative TRI_ATTN_E* code. */
 int tri_attn_uses_matrix_cores(const TriAttnArgs* args, int pass);
 
