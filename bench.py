@@ -240,8 +240,11 @@ def config_figures(dev, with_cpu):
     out = {}
     for name, wl in {**workloads.WORKLOADS, **workloads.EXTRA_WORKLOADS}.items():
         pth = Path(wl, dev)
-        # (enough warm-up steps for the clock to settle after the idle time of the CPU baseline before it)
-        ms, pk = run_steps(pth, 5 if name == "C5" else 30, 2 if name == "C5" else 8)
+        # The CPU baseline before it left the GPU idle and its clock low: warm up with this configuration's own steps for
+        # about 0.15 s (the clock needs tens of milliseconds of load), at least 8 steps, then time.
+        rough, _ = run_steps(pth, 2, 1)
+        warm = 2 if name == "C5" else max(8, min(4000, int(150.0 / max(rough, 1e-3))))
+        ms, pk = run_steps(pth, 5 if name == "C5" else 30, warm)
         peak = PEAK_TFLOPS[_dtype_name(wl.dtype)]
         f = wl.flops() / (pk["fwd"] + pk.get("mask_classes", 0.0)) / 1e9  # (the classification belongs to the forward)
         row = {"workload": describe(wl), "fwd_tflops": round(f, 2), "fwd_frac_of_peak": round(f / peak, 4),
