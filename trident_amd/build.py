@@ -47,7 +47,7 @@ BASELINE_KERNELS = {
     "mfma_fwd_kernel<__bf16, 64, 8, false, 1, false, false>": "C4 fwd",
     "delta_kernel<__bf16, 64>": "C4 delta",
     "mfma_dkdv_wide_kernel<__bf16, 64, 8, false, 1, false, false>": "C4 dK/dV",
-    "mfma_dq_kernel<__bf16, 64, 8, false, 1, false, false, false>": "C4 dQ",
+    "mfma_dq_kernel<__bf16, 64, 8, false, 1, false, false, false, false>": "C4 dQ",
     "mfma_fwd_kernel<__bf16, 128, 8, true, 0, true, false>": "C5 fwd",
     "mfma_dq_phased_kernel<__bf16, 128, true, true, true>": "C5 dQ + delta",
     "mfma_dkdv_phased_kernel<__bf16, 128, true, true, 0>": "C5 dK/dV",

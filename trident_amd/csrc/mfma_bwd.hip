@@ -41,10 +41,13 @@ __device__ __forceinline__ float mask_at(const void* mask, int64_t off) {
 // DMASK (with a mask): the kernel also writes the mask gradient dS (trident/kernel/attention.py:332-335), each lane four
 // consecutive keys of its row at a time; where the mask is broadcast over a dimension (dmask stride 0) the values are
 // added to the caller's zero-filled fp32 buffer with atomic adds instead.
-template <typename T, int D, int NW, bool CAUSAL, int MASK, bool DROPOUT, bool RAGGED = false, bool DMASK = false>
+// DELTA (no mask): the kernel also computes delta = rowsum(dO * O) of its rows from the dO rows it loads anyway, instead
+// of reading it, and stores it for the dK/dV pass, which then runs after this one (tri_attn_bwd_dq_delta).
+template <typename T, int D, int NW, bool CAUSAL, int MASK, bool DROPOUT, bool RAGGED = false, bool DMASK = false, bool DELTA = false>
 __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
     static_assert(!RAGGED || (NW == 4 && MASK == 0), "ragged lengths: 4 waves, no mask");
     static_assert(!DMASK || MASK != 0, "a mask gradient needs a mask");
+    static_assert(!DELTA || MASK == 0, "delta on the way: the variants without a mask");
     using Tile = SwzTile<D>;
     constexpr int kRows = 32 * NW;
     constexpr int kStages = 4;
@@ -87,7 +90,16 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
         gf[kk] = *reinterpret_cast<const u32x4*>(gorowp + (2 * kk + h) * 16);
     }
     float lse = p.lse[static_cast<int64_t>(bh) * p.S + qrow_ld];
-    const float dlt = p.delta[static_cast<int64_t>(bh) * p.S + qrow_ld];
+    float dlt = 0.f;
+    u32x4 of[DELTA ? KK : 1];
+    if constexpr (DELTA) {
+        // this lane holds half of its dO row (the other half is in lane ^ 32) and fetches the same half of the O row
+        const char* orowp = static_cast<const char*>(p.o) + (b * p.os[0] + hd * p.os[1] + static_cast<int64_t>(qrow_ld) * p.os[2]) * 2;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) of[kk] = *reinterpret_cast<const u32x4*>(orowp + (2 * kk + h) * 16);
+    } else {
+        dlt = p.delta[static_cast<int64_t>(bh) * p.S + qrow_ld];
+    }
     const float c = p.scale_log2;
     [[maybe_unused]] const float inv_scale = p.inv_scale;  // (a mask value joins its score before the scale: s + mask / scale)
     // Without dropout (and where the registers allow) the subtraction in dS = P (dP - delta) is left to the matrix pipe:
@@ -167,7 +179,22 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
         settle(gf[kk]);
     }
     settle(lse);
-    settle(dlt);
+    if constexpr (DELTA) {
+        float part = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            settle(of[kk]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                part = fmaf(Mma<T>::lo(of[kk][i]), Mma<T>::lo(gf[kk][i]), part);
+                part = fmaf(Mma<T>::hi(of[kk][i]), Mma<T>::hi(gf[kk][i]), part);
+            }
+        }
+        dlt = sum_xor32(part);
+        if (h == 0 && (!RAGGED || qrow < p.S)) p.delta[static_cast<int64_t>(bh) * p.S + qrow] = dlt;
+    } else {
+        settle(dlt);
+    }
     f32x16 dlt16;
     if constexpr (kDeltaInAcc) {
 #pragma unroll
@@ -1743,19 +1770,26 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_phased_kernel(const KParams 
 
 // ---------------------------------------------------------------------------------- launch
 template <typename T, int D, int NW, bool CAUSAL, int MASK>
-int launch_dq_waves(const KParams& p, hipStream_t stream) {
+int launch_dq_waves(const KParams& p, hipStream_t stream, bool with_delta = false) {
     const dim3 grid(p.B * p.H * (p.S / (32 * NW))), block(64 * NW);
     if constexpr (NW == 8 && D == 128 && MASK != kNoMask) {
         // with a mask gradient or dropout on top of a mask the 8-wave kernel does not fit its registers at D = 128 and
         // would spill to scratch memory (whose reloads are vector-memory loads that drain the tile prefetch): those
         // problems take 128-row workgroups, which fit
-        if (p.dmask != nullptr || p.thr8 > 0) return launch_dq_waves<T, D, 4, CAUSAL, MASK>(p, stream);
+        if (p.dmask != nullptr || p.thr8 > 0) return launch_dq_waves<T, D, 4, CAUSAL, MASK>(p, stream, with_delta);
         hipLaunchKernelGGL((mfma_dq_kernel<T, D, NW, CAUSAL, MASK, false>), grid, block, 0, stream, p);
     } else {
         if constexpr (MASK != kNoMask) {
             if (p.dmask != nullptr) {
                 if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dq_kernel<T, D, NW, CAUSAL, MASK, true, false, true>), grid, block, 0, stream, p);
                 else hipLaunchKernelGGL((mfma_dq_kernel<T, D, NW, CAUSAL, MASK, false, false, true>), grid, block, 0, stream, p);
+                return static_cast<int>(hipGetLastError());
+            }
+        }
+        if constexpr (MASK == kNoMask) {
+            if (with_delta) {
+                if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dq_kernel<T, D, NW, CAUSAL, MASK, true, false, false, true>), grid, block, 0, stream, p);
+                else hipLaunchKernelGGL((mfma_dq_kernel<T, D, NW, CAUSAL, MASK, false, false, false, true>), grid, block, 0, stream, p);
                 return static_cast<int>(hipGetLastError());
             }
         }
@@ -1790,13 +1824,16 @@ int launch_dq_dropout(const KParams& p, hipStream_t stream, bool with_delta) {
             return static_cast<int>(hipGetLastError());
         }
     }
-    if (with_delta) return TRI_ATTN_ESHAPE;  // (callers ask dq_fuses_delta first)
+    if (with_delta && MASK != kNoMask) return TRI_ATTN_ESHAPE;  // (callers ask mfma_dq_fuses_delta first)
     // 8 waves (256 query rows) when the sequence allows it, else 4 waves (128 rows)
-    if (p.S % 256 == 0) return launch_dq_waves<T, D, 8, CAUSAL, MASK>(p, stream);
-    if (p.S % 128 == 0) return launch_dq_waves<T, D, 4, CAUSAL, MASK>(p, stream);
+    if (p.S % 256 == 0) return launch_dq_waves<T, D, 8, CAUSAL, MASK>(p, stream, with_delta);
+    if (p.S % 128 == 0) return launch_dq_waves<T, D, 4, CAUSAL, MASK>(p, stream, with_delta);
     if constexpr (MASK == kNoMask) {  // any other length: 128-row workgroups with boundary handling
         const dim3 grid(p.B * p.H * ((p.S + 127) / 128)), block(256);
-        if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dq_kernel<T, D, 4, CAUSAL, kNoMask, true, true>), grid, block, 0, stream, p);
+        if (with_delta) {
+            if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dq_kernel<T, D, 4, CAUSAL, kNoMask, true, true, false, true>), grid, block, 0, stream, p);
+            else hipLaunchKernelGGL((mfma_dq_kernel<T, D, 4, CAUSAL, kNoMask, false, true, false, true>), grid, block, 0, stream, p);
+        } else if (p.thr8 > 0) hipLaunchKernelGGL((mfma_dq_kernel<T, D, 4, CAUSAL, kNoMask, true, true>), grid, block, 0, stream, p);
         else hipLaunchKernelGGL((mfma_dq_kernel<T, D, 4, CAUSAL, kNoMask, false, true>), grid, block, 0, stream, p);
         return static_cast<int>(hipGetLastError());
     }

@@ -141,11 +141,13 @@ bool mfma_supported(int which, int dtype, const KParams& p) {
     }
 }
 
-// The phased dQ kernel (no mask, 256-row workgroups, no dropout at D = 128) can compute delta itself.
+// Without a mask the dQ kernels compute delta themselves, from the dO rows they load anyway and the O rows (16-byte
+// aligned like the others): the phased kernel through LDS (32-bit row offsets), the others with per-lane loads.
 bool mfma_dq_fuses_delta(const KParams& p) {
-    if (p.mask != nullptr || p.S % 256 != 0) return false;
-    if (p.D < 64 || !(p.D == 64 || p.thr8 <= 0 || p.causal)) return false;  // (the phased dQ kernel's own limits)
-    return aligned16(p.o) && strides8(p.os) && tile_offsets_fit(p.os);
+    if (p.mask != nullptr) return false;
+    if (!aligned16(p.o) || !strides8(p.os)) return false;
+    const bool phased = p.D >= 64 && p.S % 256 == 0 && (p.D == 64 || p.thr8 <= 0 || p.causal);  // (as the launcher decides)
+    return !phased || tile_offsets_fit(p.os);
 }
 
 int persistent_grid(int items) {
