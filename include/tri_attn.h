@@ -143,8 +143,8 @@ int tri_attn_bwd_dkdv(const TriAttnArgs* args);
 int tri_attn_bwd_dq(const TriAttnArgs* args);
 
 /* bwd_delta and bwd_dq in one launch, for the problems whose dQ kernel can compute delta from the dO
- * rows it loads anyway (no mask, S a multiple of 256, fp16/bf16 with D in {64,128}; with dropout at
- * D = 128 only when is_causal is set): reads q,k,v,o,d_o,lse; writes delta and dq. tri_attn_bwd_dkdv, which reads delta, has to
+ * rows it loads anyway (the 16-bit matrix-core kernels without a mask: fp16/bf16, D in {32,64,128}, 16-byte
+ * aligned rows of o): reads q,k,v,o,d_o,lse; writes delta and dq. tri_attn_bwd_dkdv, which reads delta, has to
  * follow it. Returns TRI_ATTN_ENOFUSE without launching anything where it does not apply (then call
  * tri_attn_bwd_delta, tri_attn_bwd_dkdv, tri_attn_bwd_dq). The reference has the two launches only
  * (trident/operation/attention.py:161-199); tri_attn_bwd picks between the two sequences itself. */
