@@ -261,8 +261,9 @@ def config_figures(dev, with_cpu):
             logical, unique = 4.0 * B * H * S * S, 4.0 * B * S * S
             row["mask_stream"] = {k: {"logical_GBps": round(logical / pk[k] / 1e6, 1),
                                       "unique_GBps": round(unique / pk[k] / 1e6, 1)} for k in pk if k != "bwd_delta"}
-            lengths = (pth.mask[:, 0, 0] == 0).sum(-1)
-            row["masked_key_fraction"] = round(1.0 - float(lengths.float().mean()) / S, 4)
+            if not wl.dense_mask:
+                lengths = (pth.mask[:, 0, 0] == 0).sum(-1)
+                row["masked_key_fraction"] = round(1.0 - float(lengths.float().mean()) / S, 4)
             row["mask_stream"]["note"] = ("fp32 mask bytes every workgroup asks for (logical: B*H*S*S*4; unique: "
                                           "B*S*S*4, the heads of a batch share it) / kernel duration; HBM peak 8000 GB/s")
         if with_cpu and name in workloads.WORKLOADS:
@@ -507,7 +508,7 @@ def sustained_clock(dev, seconds=1.5):
 
 
 def describe(w):
-    extra = "causal" if w.is_causal else ("additive fp32 mask [B,1,S,S]" if w.masked else "plain")
+    extra = "causal" if w.is_causal else (("dense " if w.dense_mask else "") + "additive fp32 mask [B,1,S,S]" if w.masked else "plain")
     if w.dropout_p:
         extra += f" dropout {w.dropout_p}"
     return f"{w.name}: {_dtype_name(w.dtype)} {extra} B={w.B} H={w.H} S={w.S} D={w.D} {'fwd+bwd' if w.backward else 'fwd'}"

@@ -19,6 +19,7 @@ class Workload:
     D: int
     is_causal: bool = False
     masked: bool = False       # additive fp32 mask [B,1,S,S], keys >= len_b set to -inf
+    dense_mask: bool = False   # (with masked) N(0, 0.25) in every entry instead: no block of it is all zero or all -inf
     dropout_p: float = 0.0
     sigma_qkv: float = 1.0
     backward: bool = True
@@ -45,10 +46,11 @@ WORKLOADS = {
 }
 
 # Beyond the five benchmark configurations: C3's shape in fp32 (the kernels on the fp32 matrix instruction at a real
-# size) and a 16-bit problem with a small head (the same kernels on the 16-bit 32x32x8 instruction).
+# size), a 16-bit problem with head size 32, and C4's shape at D = 128 with a dense fp32 mask shared by the heads.
 EXTRA_WORKLOADS = {
     "F3": Workload("F3", torch.float32, 2, 16, 4096, 128, is_causal=True, seed=1103),
     "H32": Workload("H32", torch.bfloat16, 8, 16, 2048, 32, is_causal=True, seed=1132),
+    "M128": Workload("M128", torch.bfloat16, 8, 12, 2048, 128, masked=True, dense_mask=True, seed=1128),
 }
 
 
@@ -74,5 +76,7 @@ def make_inputs(w: Workload, B=None, H=None, S=None):
     k = (torch.randn(shape, generator=g) * w.sigma_qkv).to(w.dtype)
     v = (torch.randn(shape, generator=g) * w.sigma_qkv).to(w.dtype)
     d_o = torch.randn(shape, generator=g).to(w.dtype)
-    mask = length_mask(B, S, g)[0] if w.masked else None
+    mask = None
+    if w.masked:
+        mask = 0.5 * torch.randn(B, 1, S, S, generator=g) if w.dense_mask else length_mask(B, S, g)[0]
     return q, k, v, d_o, mask
