@@ -1145,6 +1145,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
     // (fetching delta ahead like lse, and deeper fragment rings, were measured: no gain)
     constexpr bool kRoomy = false;
     f32x4 sc_dlt[kRoomy ? 4 : 1];            // delta of the same rows
+    float sc_mk[MASK != kNoMask ? 16 : 1];   // mask values of the same rows at this lane's key
     u32x4 own_p[2], own_s[2], pp[2], ps[2];  // B operands of the accumulation
     constexpr int kAccSteps = 8 * DH, kAccRing = 4;
     u32x4 tf[kAccRing];                      // first transposed fragments of the accumulation
@@ -1156,6 +1157,16 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
         const char* sG = sQ + Tile::kBytes;
         const float* sLse = reinterpret_cast<const float*>(sG + Tile::kBytes);
         if (lt < n_local && (!CAUSAL || rb + 31 >= wkey0)) {
+            if constexpr (MASK != kNoMask) {
+                // requested before anything else of the step and used in its second part: the loads' latency, which
+                // used to stand in front of every block's arithmetic, passes behind the MFMAs and the barrier between
+                // the parts (a row of the block is 128 contiguous bytes across the lanes of a half wave). Requesting
+                // them a whole accumulation step earlier measured no better.
+                const int64_t mbase = b * p.ms[0] + hd * p.ms[1] + key;
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    sc_mk[i] = mask_at<T, MASK>(p.mask, mbase + static_cast<int64_t>(rb + c_row(i, h)) * p.ms[2]);
+            }
             const int qoff = 32 * member * Tile::kRowBytes;
             // row fragments of Q, then of dO, through a ring of kRing reads in flight
             constexpr int kRing = 4;
@@ -1207,10 +1218,8 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv_pair_kernel(const KParams p)
             }
             float mk[MASK != kNoMask ? 16 : 1];
             if constexpr (MASK != kNoMask) {
-                const int64_t mbase = b * p.ms[0] + hd * p.ms[1] + key;
 #pragma unroll
-                for (int i = 0; i < 16; ++i)
-                    mk[i] = mask_at<T, MASK>(p.mask, mbase + static_cast<int64_t>(rb + c_row(i, h)) * p.ms[2]);
+                for (int i = 0; i < 16; ++i) mk[i] = sc_mk[i];
             }
             Philox4 mine;  // the block of rows rb + 8 (lane % 4) + 4 h .. +3: this lane's share of the quad's four
             if constexpr (DROPOUT) mine = dropout_block(p, bh, (rb + 8 * (lane & 3) + 4 * h) >> 2, key >> 2);
