@@ -523,7 +523,8 @@ def test_more_items_than_compute_units(batches, heads, S, D, variant, device):
 
 
 @pytest.mark.parametrize("B,H,S,D,causal", [(8, 16, 896, 32, False), (8, 16, 2176, 32, True), (8, 16, 1024, 32, True),
-                                            (6, 16, 1152, 64, True), (8, 12, 896, 32, "mask"), (8, 12, 640, 64, "mask")])
+                                            (6, 16, 1152, 64, True), (8, 12, 896, 32, "mask"), (8, 12, 640, 64, "mask"),
+                                            (8, 12, 1024, 128, "mask"), (6, 12, 768, 128, True)])
 def test_a_head_does_not_depend_on_its_company(B, H, S, D, causal, device):
     """Several workgroups resident per compute unit (small heads: four 4-wave workgroups): every head of a launch with a
     thousand workgroups gets bit for bit what it gets in a launch of its batch alone, and two heads match the oracle.
