@@ -143,7 +143,7 @@ int tri_attn_bwd_dkdv(const TriAttnArgs* args);
 int tri_attn_bwd_dq(const TriAttnArgs* args);
 
 /* bwd_delta and bwd_dq in one launch, for the problems whose dQ kernel can compute delta from the dO
- * rows it loads anyway (the 16-bit matrix-core kernels without a mask: fp16/bf16, D in {32,64,128}, 16-byte
+ * rows it loads anyway (the 16-bit matrix-core kernels without a mask: fp16/bf16, D in {16,32,64,128}, 16-byte
  * aligned rows of o): reads q,k,v,o,d_o,lse; writes delta and dq. tri_attn_bwd_dkdv, which reads delta, has to
  * follow it. Returns TRI_ATTN_ENOFUSE without launching anything where it does not apply (then call
  * tri_attn_bwd_delta, tri_attn_bwd_dkdv, tri_attn_bwd_dq). The reference has the two launches only
@@ -183,10 +183,10 @@ int64_t tri_attn_mask_classes_size(const TriAttnArgs* args);
 
 /* Which kernel family a call would run, without launching anything (no counterpart in the reference): pass 0 =
  * tri_attn_fwd, 1 = tri_attn_bwd_dkdv, 2 = tri_attn_bwd_dq on these arguments. Returns 1 for the 16-bit matrix-core
- * (MFMA) kernels (fp16/bf16, D in {32,64,128}, 16-byte aligned rows; any S without a mask, S a multiple of 128 with
+ * (MFMA) kernels (fp16/bf16, D in {16,32,64,128}, 16-byte aligned rows; any S without a mask, S a multiple of 128 with
  * one); 2 for the 32-row-tile matrix-core kernels (everything else whose pointers and strides are multiples of
  * four elements: fp32 problems on the fp32 matrix instruction with fp32 products and sums; fp16/bf16 problems with
- * D = 16 or masked lengths that are no multiple of 128 on the 16-bit 32x32x8 instruction);
+ * masked lengths that are no multiple of 128 on the 16-bit 32x32x8 instruction);
  * 0 for the general vector-ALU kernels (views that are not aligned so); or a negative TRI_ATTN_E* code. */
 int tri_attn_uses_matrix_cores(const TriAttnArgs* args, int pass);
 

@@ -188,7 +188,7 @@ def test_key_padding_mask_row_broadcast(dtype, D, S, p, device):
                                                      (torch.float16, torch.float16, (1, 3, 256, 256)),
                                                      (torch.bfloat16, torch.float32, (2, 1, 1, 256)),
                                                      (torch.float32, torch.float32, (1, 1, 1, 256))])
-@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("D", [16, 32, 64, 128])
 def test_mask_gradient_on_the_matrix_cores(dtype, mask_dtype, mshape, D, device):
     """The mask gradient from the matrix-core dQ kernel (16-bit problems): written in place for a full mask, added
     atomically into the mask's own shape for masks broadcast over batch, heads or rows (a key-padding mask with a
@@ -362,7 +362,7 @@ def _abi_case(device, dtype, S, D, variant, seed, batches=1, heads=2, matrix_cor
 
 
 @pytest.mark.parametrize("variant", ["plain", "causal", "mask", "mask16", "causal+dropout"])
-@pytest.mark.parametrize("S,D", [(384, 64), (384, 128), (640, 64), (640, 128), (384, 32), (640, 32)])
+@pytest.mark.parametrize("S,D", [(384, 64), (384, 128), (640, 64), (640, 128), (384, 32), (640, 32), (384, 16), (1024, 16)])
 def test_four_wave_kernels_over_several_tiles(S, D, variant, device):
     _abi_case(device, torch.bfloat16, S, D, variant, 200 + S + D)
 
@@ -409,7 +409,7 @@ def test_operator_without_the_reference_limits(dtype, S, D, device):
                                        (torch.float16, 72, 64), (torch.bfloat16, 200, 128), (torch.bfloat16, 129, 64),
                                        (torch.float16, 255, 128), (torch.bfloat16, 1000, 64), (torch.bfloat16, 1, 64),
                                        (torch.float16, 833, 128), (torch.bfloat16, 32, 32), (torch.float16, 333, 32),
-                                       (torch.bfloat16, 1, 32)])
+                                       (torch.bfloat16, 1, 32), (torch.float16, 70, 16), (torch.bfloat16, 333, 16)])
 def test_any_length_runs_on_the_matrix_cores(dtype, S, D, variant, device):
     """Lengths that are not multiples of 128 (the reference's benchmark regime S = 32, 64 among them): the 128-row
     matrix-core kernels with boundary handling (clamped loads, masked keys and rows, guarded stores), not the
@@ -418,11 +418,12 @@ def test_any_length_runs_on_the_matrix_cores(dtype, S, D, variant, device):
 
 
 def test_what_the_16_bit_kernels_leave_runs_on_the_32_row_tile_kernels(device):
-    """Masked problems of other lengths, fp32 problems and the smallest head: family 2 (v_mfma_f32_32x32x2_f32 for fp32
-    data, the 16-bit 32x32x8 instruction for 16-bit data) in all three passes; a 16-bit head of 32 is family 1."""
+    """Masked problems of other lengths and fp32 problems: family 2 (v_mfma_f32_32x32x2_f32 for fp32 data, the 16-bit
+    32x32x8 instruction for 16-bit data) in all three passes; 16-bit heads of 16 and 32 are family 1."""
     _abi_case(device, torch.bfloat16, 200, 64, "mask", 650, matrix_cores=[2, 2, 2])
     _abi_case(device, torch.float32, 256, 64, "plain", 651, matrix_cores=[2, 2, 2])
-    _abi_case(device, torch.bfloat16, 256, 16, "causal", 652, matrix_cores=[2, 2, 2])
+    _abi_case(device, torch.bfloat16, 200, 16, "mask", 654, matrix_cores=[2, 2, 2])
+    _abi_case(device, torch.bfloat16, 256, 16, "causal", 652, matrix_cores=[1, 1, 1])
     _abi_case(device, torch.bfloat16, 256, 32, "causal", 653, matrix_cores=[1, 1, 1])
 
 
@@ -437,8 +438,8 @@ def test_32_row_tile_kernels(dtype, S, D, variant, device):
     size, over lengths with a ragged last tile (and one of a single row), three heads, every mask mode and dropout."""
     if variant == "mask16" and dtype == torch.float32:
         pytest.skip("a 16-bit mask is a mask of the operand type")
-    # (a 16-bit head of 32 without a mask is the 64-key-tile kernels' at any length)
-    family = 1 if dtype != torch.float32 and D == 32 and "mask" not in variant else 2
+    # (16-bit heads of 16 and 32 without a mask are the 64-key-tile kernels' at any length)
+    family = 1 if dtype != torch.float32 and D <= 32 and "mask" not in variant else 2
     _abi_case(device, dtype, S, D, variant, 700 + S + D, batches=2 if S < 300 else 1, heads=3, matrix_cores=[family] * 3)
 
 
@@ -524,6 +525,7 @@ def test_more_items_than_compute_units(batches, heads, S, D, variant, device):
 
 @pytest.mark.parametrize("B,H,S,D,causal", [(8, 16, 896, 32, False), (8, 16, 2176, 32, True), (8, 16, 1024, 32, True),
                                             (6, 16, 1152, 64, True), (8, 12, 896, 32, "mask"), (8, 12, 640, 64, "mask"),
+                                            (8, 16, 1152, 16, True), (8, 12, 896, 16, "mask"),
                                             (8, 12, 1024, 128, "mask"), (6, 12, 768, 128, True)])
 def test_a_head_does_not_depend_on_its_company(B, H, S, D, causal, device):
     """Several workgroups resident per compute unit (small heads: four 4-wave workgroups): every head of a launch with a

@@ -1,4 +1,4 @@
-// Backward attention on the matrix cores for fp16/bf16, D in {32,64,128}, S a multiple of 128
+// Backward attention on the matrix cores for fp16/bf16, D in {16,32,64,128}, S a multiple of 128
 // (replaces trident/kernel/attention.py:169-339, split in two passes so that no gradient
 // tile is ever accumulated in global memory):
 //
@@ -53,7 +53,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
     constexpr int kStages = 4;
     constexpr int kStageBytes = 2 * Tile::kBytes;  // K tile, V tile
     constexpr int KK = D / 16;
-    constexpr int DB = D / 32;
+    constexpr int DB = D >= 32 ? D / 32 : 1;  // (D = 16: one block of gradient columns, the upper 16 are not stored)
     constexpr int kBlocksPerWave = 2 * Tile::kBlocks / NW;  // LDS-direct loads per wave and tile
     static_assert(2 * Tile::kBlocks % NW == 0, "tile blocks must divide among the waves");
     // A mask block of a wave (32 rows x 64 keys) goes through a private LDS region (8 KiB fp32, 4 KiB for a mask of
@@ -348,7 +348,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_dq_kernel(const KParams p) {
     // every wave is out of the loop: the ring can serve as the waves' private transposition patches
     lds_barrier();
     {
-        using Store = RowBlockStore<T, DB>;
+        using Store = RowBlockStore<T, DB, D < 32 ? D : 32 * DB>;
         static_assert(NW * Store::kPatchBytes <= kStages * kStageBytes, "patches must fit into the ring");
         char* out0 = static_cast<char*>(p.dq) + (b * p.dqs[0] + hd * p.dqs[1] + static_cast<int64_t>(wrow0) * p.dqs[2]) * 2;
         const float sc = kDeltaInAcc ? -p.scale : p.scale;
@@ -664,7 +664,7 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
     constexpr int kStages = 4;
     constexpr int kStageBytes = 2 * Tile::kBytes + 2 * kBN * 4;  // Q tile, dO tile, lse, delta
     constexpr int KK = D / 16;
-    constexpr int DB = D / 32;
+    constexpr int DB = D >= 32 ? D / 32 : 1;  // (D = 16: one block of gradient columns, the upper 16 are not stored)
     constexpr int kBlocksPerWave = 2 * Tile::kBlocks / NW;
     constexpr int kLoadsPerTile = kBlocksPerWave + 1;            // + lse or delta: exact for every wave
     static_assert(2 * Tile::kBlocks % NW == 0, "tile blocks must divide among the waves");
@@ -962,7 +962,7 @@ __global__ __launch_bounds__(NW * 64, RAGGED ? 1 : 2) void mfma_dkdv_wide_kernel
     // every wave is out of the loop: the ring can serve as the waves' private transposition patches
     lds_barrier();
     {
-        using Store = RowBlockStore<T, DB>;
+        using Store = RowBlockStore<T, DB, D < 32 ? D : 32 * DB>;
         static_assert(NW * Store::kPatchBytes <= kStages * kStageBytes, "patches must fit into the ring");
         char* patch = smem + wave * Store::kPatchBytes;
         char* dk0 = static_cast<char*>(p.dk) + (b * p.dks[0] + hd * p.dks[1] + static_cast<int64_t>(wkey0) * p.dks[2]) * 2;
@@ -1846,7 +1846,9 @@ int launch_dq_dropout(const KParams& p, hipStream_t stream, bool with_delta) {
     }
     if (with_delta && MASK != kNoMask) return TRI_ATTN_ESHAPE;  // (callers ask mfma_dq_fuses_delta first)
     // 8 waves (256 query rows) when the sequence allows it, else 4 waves (128 rows)
-    if (p.S % 256 == 0) return launch_dq_waves<T, D, 8, CAUSAL, MASK>(p, stream, with_delta);
+    if constexpr (D > 16) {  // (a D = 16 tile has four blocks in all: four waves)
+        if (p.S % 256 == 0) return launch_dq_waves<T, D, 8, CAUSAL, MASK>(p, stream, with_delta);
+    }
     if (p.S % 128 == 0) return launch_dq_waves<T, D, 4, CAUSAL, MASK>(p, stream, with_delta);
     if constexpr (MASK == kNoMask) {  // any other length: 128-row workgroups with boundary handling
         const dim3 grid(p.B * p.H * ((p.S + 127) / 128)), block(256);
@@ -1884,7 +1886,9 @@ int launch_dkdv_dropout(const KParams& p, hipStream_t stream) {
     if constexpr (D <= 64) {
         // the two-waves-per-SIMD kernel fits its registers: 8 waves (256 keys) when the sequence
         // allows it, else 4 waves (128 keys)
-        if (p.S % 256 == 0) return launch_dkdv_waves<T, D, 8, CAUSAL, MASK>(p, stream);
+        if constexpr (D > 16) {
+            if (p.S % 256 == 0) return launch_dkdv_waves<T, D, 8, CAUSAL, MASK>(p, stream);
+        }
         return launch_dkdv_waves<T, D, 4, CAUSAL, MASK>(p, stream);
     } else {
         // D = 128: K, V and both gradient accumulators of a 32-key block take 192 registers, too many
@@ -1931,7 +1935,8 @@ template <int WHICH, typename T>
 int launch_bwd_head(int dtype, const KParams& p, hipStream_t stream, bool with_delta) {
     if (p.D == 128) return launch_bwd_variant<WHICH, T, 128>(dtype, p, stream, with_delta);
     if (p.D == 64) return launch_bwd_variant<WHICH, T, 64>(dtype, p, stream, with_delta);
-    return launch_bwd_variant<WHICH, T, 32>(dtype, p, stream, with_delta);
+    if (p.D == 32) return launch_bwd_variant<WHICH, T, 32>(dtype, p, stream, with_delta);
+    return launch_bwd_variant<WHICH, T, 16>(dtype, p, stream, with_delta);
 }
 
 template <int WHICH>

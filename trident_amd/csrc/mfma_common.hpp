@@ -176,6 +176,7 @@ struct SwzTile {
     static __device__ __forceinline__ int swz(int r) {
         if constexpr (D == 128) return ((r & 7) << 1) | ((r >> 3) & 1);
         else if constexpr (D == 32) return (r >> 2) & 3;  // (64-byte rows, four chunks: four rows fill the 64 banks once)
+        else if constexpr (D == 16) return (r >> 3) & 1;  // (32-byte rows, two chunks: eight rows fill the banks once)
         else return (((r >> 1) & 3) << 1) | ((r >> 3) & 1);
     }
     static __device__ __forceinline__ int off(int r, int c) { return r * kRowBytes + ((c ^ swz(r)) << 4); }
@@ -199,7 +200,8 @@ struct SwzTile {
     static __device__ __forceinline__ int tr_off(int db, int half, int lane) {
         const int g = lane >> 4, lam = lane & 15;
         const int r = 8 * half + 4 * (g >> 1) + (lam >> 2);
-        const int col = 32 * db + 16 * (g & 1) + 4 * (lam & 3);
+        // (D = 16: a row has 16 columns; the lanes of the upper 16 repeat the lower ones, their products are not stored)
+        const int col = 32 * db + (D > 16 ? 16 * (g & 1) : 0) + 4 * (lam & 3);
         return r * kRowBytes + (((col >> 3) ^ swz(r)) << 4) + ((lam & 1) << 3);
     }
     static __device__ __forceinline__ u32x4 tr_frag(const char* tile, int off_half0, int off_half1, int ks) {
@@ -323,9 +325,10 @@ __device__ __forceinline__ TileClasses tile_classes(const uint8_t* first, int64_
 // lane along the rows, so that a store instruction writes whole 64 NB-byte row segments.
 // `patch` must be private to the wave and no longer in use by anyone (barrier before the call).
 // `scale(i)` is applied per register; `row0` points at column 0 of the wave's first row.
-template <typename T, int NB>
+// COLS < 32 NB: only the first COLS columns of the block exist and are stored (head size 16: one block, 16 columns).
+template <typename T, int NB, int COLS = 32 * NB>
 struct RowBlockStore {
-    static constexpr int kRowBytes = 64 * NB;
+    static constexpr int kRowBytes = 2 * COLS;
     static constexpr int kPitch = kRowBytes + 16;
     static constexpr int kPatchBytes = 32 * kPitch;
     static constexpr int kLanesPerRow = kRowBytes / 16;
@@ -339,6 +342,7 @@ struct RowBlockStore {
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
+                if (32 * nb + 8 * g >= COLS) continue;  // (columns that do not exist)
                 u32x2 v;
                 v.x = Mma<T>::pack2(scale(acc[nb][4 * g + 0]), scale(acc[nb][4 * g + 1]));
                 v.y = Mma<T>::pack2(scale(acc[nb][4 * g + 2]), scale(acc[nb][4 * g + 3]));

@@ -1,5 +1,5 @@
 // Forward attention on the matrix cores: online-softmax flash kernel for fp16/bf16,
-// D in {32,64,128}; any S without a mask, multiples of 128 with one (replaces trident/kernel/attention.py:33-165).
+// D in {16,32,64,128}; any S without a mask, multiples of 128 with one (replaces trident/kernel/attention.py:33-165).
 //
 // A workgroup of NW waves owns 32*NW query rows, one wave 32 of them. Q stays in registers as
 // the B operand of S^T = K Q^T; K and V tiles of 64 keys live row-major (swizzled) in a four-stage
@@ -55,13 +55,13 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     constexpr int kBlocksPerWave = 2 * Tile::kBlocks / NW;  // LDS-direct loads per wave and tile
     static_assert(kBlocksPerWave >= 1, "every wave fetches a piece of every tile");
     constexpr int KK = D / 16;  // K-steps of S^T
-    constexpr int DB = D / 32;  // 32-row blocks of O^T
+    constexpr int DB = D >= 32 ? D / 32 : 1;  // 32-row blocks of O^T (D = 16: one block whose upper 16 rows are not stored)
     constexpr int kSteps = 2 * KK;    // MFMAs of S^T per tile
     constexpr int kPvSteps = 4 * DB;  // MFMAs of O^T per tile
     // operand fragments in flight (a mask and dropout together at D = 128 leave room for four only)
     // (at D = 32 the O^T product has four steps, and the softmax phase may request fragments of tile j only: tile j + 1
     // becomes visible with the barrier behind it)
-    constexpr int kRing = (D == 32 || (D == 128 && MASK != kNoMask && DROPOUT)) ? 4 : 6;
+    constexpr int kRing = (D <= 32 || (D == 128 && MASK != kNoMask && DROPOUT)) ? 4 : 6;
     static_assert(kRing <= kPvSteps, "the softmax phase requests fragments of the O^T product only");
     // A mask block of a wave (32 rows x 64 keys) goes through a private LDS region (8 KiB for an fp32 mask, 4 KiB
     // for one of the operand type) when it fits (D = 64): lanes own rows, so direct loads would touch 32 cache
@@ -77,7 +77,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     // passes behind the epilogue. The epilogue's transposition patches then must not lie in ring stages 0-2.
     constexpr bool kPersistent = NW == 8 && MASK == kNoMask;
     constexpr int kStoreBlocks = DB >= 2 ? 2 : 1;
-    using Store = RowBlockStore<T, kStoreBlocks>;            // the epilogue stores 64 columns at a time (32 at D = 32)
+    using Store = RowBlockStore<T, kStoreBlocks, D < 32 ? D : 32 * kStoreBlocks>;  // the epilogue stores 64 columns at a time (32 at D = 32, 16 at D = 16)
     constexpr int kPatchOff = kPersistent ? kVRing + 3 * Tile::kBytes : 0;  // (behind the V tile of slot 2)
     constexpr int kRingBytes = kStages * kStageBytes;
     constexpr int kPatchEnd = kPatchOff + NW * Store::kPatchBytes;
@@ -155,16 +155,31 @@ __global__ __launch_bounds__(NW * 64, 2) void mfma_fwd_kernel(const KParams p) {
     // A wave fetches blocks wave, wave + NW, ... of the K tile and of the V tile: their rows are a
     // multiple of 16 apart, so one per-lane source offset (row within the block, swizzled chunk)
     // serves all of them and the rest of the address is scalar arithmetic.
-    constexpr int kPerOperand = Tile::kBlocks / NW;
+    // (D = 16 with 4 waves: a tile has two blocks per operand, waves 0-1 fetch the K tile's and waves 2-3 the V tile's)
+    constexpr bool kSplitOperands = Tile::kBlocks < NW;
+    constexpr int kPerOperand = kSplitOperands ? 1 : Tile::kBlocks / NW;
     constexpr int kRowStep = NW * Tile::kRowsPerBlock;
-    static_assert(kPerOperand >= 1 && kRowStep % 16 == 0 && 2 * kPerOperand == kBlocksPerWave, "block assignment");  // (D = 32: 4 waves)
-    const uint32_t koff = static_cast<uint32_t>(Tile::src_off(wave, lane, krow_bytes));
-    const uint32_t voff = static_cast<uint32_t>(Tile::src_off(wave, lane, vrow_bytes));
+    static_assert(kRowStep % 16 == 0 && (kSplitOperands ? kBlocksPerWave == 1 && 2 * Tile::kBlocks == NW && !kLeadK
+                                                        : 2 * kPerOperand == kBlocksPerWave), "block assignment");
+    const int my_block = kSplitOperands ? wave % Tile::kBlocks : wave;
+    const uint32_t koff = static_cast<uint32_t>(Tile::src_off(my_block, lane, krow_bytes));
+    const uint32_t voff = static_cast<uint32_t>(Tile::src_off(my_block, lane, vrow_bytes));
     // load number idx (0 .. kBlocksPerWave-1) of this wave's share of the K tile t (the first kPerOperand) and of the V
     // tile t - kLag (the others) -> ring slot (tile % kStages) of the operand
     auto issue_load = [&](int tk, int idx) {
         const int t = idx < kPerOperand ? tk : tk - kLag;
-        char* stage = smem + (t % kStages) * kKBytes + wave * 1024;
+        char* stage = smem + (t % kStages) * kKBytes + my_block * 1024;
+        if constexpr (kSplitOperands) {  // (this wave's one load: a block of the K tile or of the V tile)
+            const int last = p.S - 1 - t * kBN;
+            const bool partial = RAGGED && (t + 1) * kBN > p.S;
+            if (wave < Tile::kBlocks)
+                lds_direct_load16(kbase + static_cast<int64_t>(t) * kBN * krow_bytes,
+                                  partial ? Tile::src_off_clamped(my_block, lane, krow_bytes, last) : koff, stage);
+            else
+                lds_direct_load16(vbase + static_cast<int64_t>(t) * kBN * vrow_bytes,
+                                  partial ? Tile::src_off_clamped(my_block, lane, vrow_bytes, last) : voff, stage + kVRing);
+            return;
+        }
         const int i = idx % kPerOperand;
         if (RAGGED && (t + 1) * kBN > p.S) {  // the sequence ends inside this tile: clamped rows, offsets from the tile's first row
             const int last = p.S - 1 - t * kBN;
@@ -624,7 +639,7 @@ int launch_fwd_waves(int dtype, const KParams& p, hipStream_t stream) {
     // 8 waves (256 query rows) when the sequence allows it: two waves per SIMD out of phase. At D = 32 the vector ALU
     // is the busy unit and a workgroup's phases are short: four independent 4-wave workgroups per CU (the kernel then
     // fits 128 registers) measured 28 % faster than the 8-wave pairs.
-    if constexpr (D != 32) {
+    if constexpr (D > 32) {
         if (p.S % 256 == 0) return launch_fwd_variant<T, D, 8>(dtype, p, stream);
     }
     if (p.S % 128 == 0) return launch_fwd_variant<T, D, 4>(dtype, p, stream);
@@ -636,7 +651,8 @@ template <typename T>
 int launch_fwd_head(int dtype, const KParams& p, hipStream_t stream) {
     if (p.D == 128) return launch_fwd_waves<T, 128>(dtype, p, stream);
     if (p.D == 64) return launch_fwd_waves<T, 64>(dtype, p, stream);
-    return launch_fwd_waves<T, 32>(dtype, p, stream);
+    if (p.D == 32) return launch_fwd_waves<T, 32>(dtype, p, stream);
+    return launch_fwd_waves<T, 16>(dtype, p, stream);
 }
 
 }  // namespace

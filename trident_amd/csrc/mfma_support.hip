@@ -14,7 +14,7 @@ bool strides8(const int64_t* s) { return (s[0] % 8) == 0 && (s[1] % 8) == 0 && (
 // Pure streaming: 16-byte loads, D/8 lanes per row, fp32 accumulation, one fp32 store per row.
 template <typename T, int D>
 __global__ __launch_bounds__(256) void delta_kernel(const KParams p) {
-    constexpr int kLanes = D / 8;           // lanes per row: 16 (D=128), 8 (D=64) or 4 (D=32)
+    constexpr int kLanes = D / 8;           // lanes per row: 16 (D=128), 8 (D=64), 4 (D=32) or 2 (D=16)
     constexpr int kRowsPerBlock = 256 / kLanes;
     const int sub = threadIdx.x % kLanes;
     const int64_t row_lin = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + threadIdx.x / kLanes;
@@ -106,7 +106,7 @@ static bool tile_offsets_fit(const int64_t* strides) { return strides[2] >= 0 &&
 
 bool mfma_supported(int which, int dtype, const KParams& p) {
     if (dtype != TRI_ATTN_F16 && dtype != TRI_ATTN_BF16) return false;
-    if (p.D != 32 && p.D != 64 && p.D != 128) return false;
+    if (p.D != 16 && p.D != 32 && p.D != 64 && p.D != 128) return false;
     // lengths that are not multiples of 128 run the 4-wave kernels with boundary handling; those read no mask
     if (p.S % 128 != 0 && p.mask != nullptr) return false;
     if (!(p.scale > 0.f)) return false;  // the kernels take row maxima before scaling
@@ -163,13 +163,15 @@ int persistent_grid(int items) {
 }
 
 int launch_delta(int dtype, const KParams& p, hipStream_t stream) {
-    const bool vec = (dtype == TRI_ATTN_F16 || dtype == TRI_ATTN_BF16) && (p.D == 32 || p.D == 64 || p.D == 128) &&
+    const bool vec = (dtype == TRI_ATTN_F16 || dtype == TRI_ATTN_BF16) && (p.D == 16 || p.D == 32 || p.D == 64 || p.D == 128) &&
                      aligned16(p.o) && aligned16(p.d_o) && strides8(p.os) && strides8(p.dos) &&
                      (static_cast<int64_t>(p.B) * p.H * p.S) % 128 == 0;
     if (!vec) return launch_generic_any(kGenericDelta, dtype, p, stream);
     if (dtype == TRI_ATTN_BF16)
-        return p.D == 128 ? launch_delta_t<bf16_t, 128>(p, stream) : p.D == 64 ? launch_delta_t<bf16_t, 64>(p, stream) : launch_delta_t<bf16_t, 32>(p, stream);
-    return p.D == 128 ? launch_delta_t<f16_t, 128>(p, stream) : p.D == 64 ? launch_delta_t<f16_t, 64>(p, stream) : launch_delta_t<f16_t, 32>(p, stream);
+        return p.D == 128 ? launch_delta_t<bf16_t, 128>(p, stream) : p.D == 64 ? launch_delta_t<bf16_t, 64>(p, stream)
+             : p.D == 32 ? launch_delta_t<bf16_t, 32>(p, stream) : launch_delta_t<bf16_t, 16>(p, stream);
+    return p.D == 128 ? launch_delta_t<f16_t, 128>(p, stream) : p.D == 64 ? launch_delta_t<f16_t, 64>(p, stream)
+         : p.D == 32 ? launch_delta_t<f16_t, 32>(p, stream) : launch_delta_t<f16_t, 16>(p, stream);
 }
 
 }  // namespace tri
