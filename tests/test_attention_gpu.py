@@ -145,7 +145,7 @@ def test_shapes(dtype, S, D, variant, device):
 @pytest.mark.parametrize("S,D,causal", [(256, 64, True), (512, 128, False), (200, 128, True), (333, 32, False)])
 def test_strided_inputs(dtype, S, D, causal, device):
     """[B,S,H,D] storage viewed as [B,H,S,D]: rows of one head are H*D apart. Through the phased 16-bit kernels, their
-    variants for other lengths, and the 32-row-tile kernels (fp32; head size 32)."""
+    variants for other lengths, and the 32-row-tile kernels (fp32)."""
     B, H = 2, 4
     g = torch.Generator().manual_seed(21)
     q, k, v, d_o = [torch.randn(B, S, H, D, generator=g).to(dtype).transpose(1, 2) for _ in range(4)]

@@ -1,6 +1,6 @@
 // Attention on 32-row tiles, four waves to a workgroup: fp32 inputs (on the fp32 matrix instruction,
-// v_mfma_f32_32x32x2_f32), and every 16-bit problem the 16-bit kernels proper do not take (head sizes 16 and 32, masked
-// lengths that are not multiples of 128; on v_mfma_f32_32x32x8_{f16,bf16_1k}). Any S >= 1, D in {16, 32, 64, 128},
+// v_mfma_f32_32x32x2_f32), and every 16-bit problem the 16-bit kernels proper do not take (masked lengths that are not
+// multiples of 128, rows aligned to four elements only; on v_mfma_f32_32x32x8_{f16,bf16_1k}). Any S >= 1, D in {16, 32, 64, 128},
 // fp32 / fp16 / bf16 storage, additive mask of any dtype and broadcast, causal mask, dropout.
 // With fp32 data products and sums are fp32 throughout (the instruction multiplies fp32 exactly), so results agree with
 // the vector-ALU kernels of generic.hip to rounding; those remain for views whose rows are not 4-element aligned. With
