@@ -46,10 +46,11 @@ WORKLOADS = {
 }
 
 # Beyond the five benchmark configurations: C3's shape in fp32 (the kernels on the fp32 matrix instruction at a real
-# size), a 16-bit problem with head size 32, and C4's shape at D = 128 with a dense fp32 mask shared by the heads.
+# size), 16-bit problems with head sizes 32 and 16, and C4's shape at D = 128 with a dense fp32 mask shared by the heads.
 EXTRA_WORKLOADS = {
     "F3": Workload("F3", torch.float32, 2, 16, 4096, 128, is_causal=True, seed=1103),
     "H32": Workload("H32", torch.bfloat16, 8, 16, 2048, 32, is_causal=True, seed=1132),
+    "H16": Workload("H16", torch.bfloat16, 8, 16, 2048, 16, is_causal=True, seed=1116),
     "M128": Workload("M128", torch.bfloat16, 8, 12, 2048, 128, masked=True, dense_mask=True, seed=1128),
 }
 
